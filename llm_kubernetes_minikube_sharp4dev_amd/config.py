@@ -127,6 +127,8 @@ class ModelPresets:
         "llama-tiny": "llama-tiny",
         "lebepel-tiny": "lebepel-tiny",
         "lebepel-1b": "lebepel-1b",
+        "fusasun-tiny": "fusasun-tiny",
+        "fusasun-1b": "fusasun-1b",
     })
     embedders: dict = field(default_factory=lambda: {
         "nomic-embed-text": "nomic-embed-text",

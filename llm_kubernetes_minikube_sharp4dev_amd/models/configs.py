@@ -181,6 +181,81 @@ class PemidraConfig:
                            for l in self.layers]}
 
 
+
+@dataclass
+class FusasunConfig:
+    """The Fusasun design: an f32 residual stream, every sublayer normed before and after
+    (``x += rms(gate * sub(rms(x) w_pre)) w_post`` with the gate ``sigmoid(W_rg h + b)`` of the sublayer's
+    input), a short causal convolution added to what the mixer reads (``canon_taps`` taps per channel, its
+    last inputs part of a sequence's state), two sliding-window mixers in any order -- ``attention``
+    (grouped-query, pooled blocks before the window) and ``latent_attention`` -- and a feed-forward of
+    experts chosen by the token id from a table.  The embedding is multiplied by ``embed_scale``.
+    Every size and constant comes from the checkpoint's ``config.json`` (:meth:`from_json`)."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layers: list                 # [HybridLayer]
+    norm_eps: float = 1e-6
+    embed_scale: float = 1.0
+    canon_taps: int = 1
+    max_position: int = 1 << 20  # nothing in the design bounds a sequence; engines pass their own limit
+    arch: str = "fusasun"
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    tie_word_embeddings: bool = False
+
+    MIXERS = ("attention", "latent_attention")
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_json(cls, d: dict, name: str = "fusasun") -> "FusasunConfig":
+        layers = [HybridLayer(l["type"], dict(l["mixer"]), dict(l["mlp"]) if l.get("mlp") else None)
+                  for l in d["layers"]]
+        for l in layers:
+            if l.type not in cls.MIXERS:
+                raise ValueError(f"unknown mixer type {l.type!r}")
+            if l.mlp is not None and l.mlp.get("kind", "moe") != "moe":
+                raise ValueError(f"unknown feed-forward kind {l.mlp.get('kind')!r}")
+        taps = int((d.get("canon") or {}).get("taps", 1))
+        if not 1 <= taps <= 8:
+            raise ValueError(f"canon.taps {taps} outside 1..8")
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=layers,
+                   norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)),
+                   embed_scale=float((d.get("embedding") or {}).get("scale", 1.0)), canon_taps=taps,
+                   max_position=int(d.get("max_positions", 1 << 20)))
+
+    def to_json(self) -> dict:
+        return {"architecture": "Fusasun", "vocab": self.vocab_size, "width": self.hidden, "norm": {"eps": self.norm_eps},
+                "embedding": {"scale": self.embed_scale}, "canon": {"taps": self.canon_taps},
+                "layers": [{"type": l.type, "mixer": dict(l.mixer), "mlp": dict(l.mlp) if l.mlp else None}
+                           for l in self.layers]}
+
+
+def fusasun_layers(n: int, heads: int, head_dim: int, ff: int, experts: int, top: int, kv_heads: Optional[int] = None,
+                   window: int = 1024, pool: int = 64, rot_dim: int = 64, q_rank: int = 768, kv_rank: int = 256,
+                   pattern=("attention", "latent_attention"), original: int = 8192) -> list:
+    """``n`` layers cycling through ``pattern`` with one set of head sizes (presets and benchmarks)."""
+    kv = kv_heads or heads
+    out = []
+    for i in range(n):
+        t = pattern[i % len(pattern)]
+        if t == "attention":
+            mixer = {"heads": heads, "kv_heads": kv, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                     "mask": {"size": window, "pool": pool},
+                     "rot": {"base": 500000.0, "dims": head_dim,
+                             "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": original}}}
+        else:
+            mixer = {"heads": heads, "dim": head_dim, "rot_dim": rot_dim, "vdim": head_dim, "q_rank": q_rank, "kv_rank": kv_rank,
+                     "scale": (head_dim + rot_dim) ** -0.5, "mask": {"size": window},
+                     "rot": {"base": 10000.0, "dims": rot_dim,
+                             "scaling": {"factor": 4.0, "original": original, "fast": 32.0, "slow": 1.0}}}
+        out.append(HybridLayer(t, mixer, {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+                               if ff else None))
+    return out
+
 def pemidra_layers(n: int, heads: int, head_dim: int, ff: int, kv_heads: Optional[int] = None, chunk: int = 256,
                    rot_dims: Optional[int] = None, lora: int = 128, conv: int = 4,
                    pattern=("general_delta", "retention", "parallel")) -> list:
@@ -259,6 +334,15 @@ DECODERS.update({
     "pemidra-1b": PemidraConfig("pemidra-1b", 32768, 2048, pemidra_layers(18, 16, 128, 5632, kv_heads=4), postln_alpha=2.0),
 })
 
+DECODERS.update({
+    # pooled-window / latent attention decoders with table-routed experts (random-init presets)
+    "fusasun-tiny": FusasunConfig("fusasun-tiny", 32768, 128, fusasun_layers(3, 4, 24, 40, 6, 2, kv_heads=2, window=20, pool=6,
+                                                                              rot_dim=8, q_rank=48, kv_rank=40, original=64),
+                                  embed_scale=2.0, canon_taps=4),
+    "fusasun-1b": FusasunConfig("fusasun-1b", 32768, 2048, fusasun_layers(16, 16, 128, 512, 16, 2, kv_heads=4),
+                                embed_scale=1.0, canon_taps=4),
+})
+
 ENCODERS = {
     "bge-base": EncoderConfig("bge-base", "bert", 12, 768, 12, 3072, 30522, pooling="cls"),
     "minilm-l6": EncoderConfig("minilm-l6", "bert", 6, 384, 12, 1536, 30522, pooling="mean"),
@@ -286,6 +370,20 @@ def encoder_config(name: str, **overrides) -> EncoderConfig:
 
 
 def param_count(cfg) -> int:
+    if isinstance(cfg, FusasunConfig):
+        W, n = cfg.hidden, 2 * cfg.vocab_size * cfg.hidden + cfg.hidden
+        for l in cfg.layers:
+            m = l.mixer
+            if l.type == "attention":
+                n += W * (m["heads"] * (m["dim"] + m["vdim"]) + m["kv_heads"] * (m["dim"] + m["vdim"]))
+            else:
+                qd = m["dim"] + m["rot_dim"]
+                n += W * (m["q_rank"] + m["kv_rank"] + m["rot_dim"] + m["heads"]) + m["q_rank"] * (1 + m["heads"] * qd) \
+                    + m["kv_rank"] * (1 + m["heads"] * (m["dim"] + m["vdim"])) + W * m["heads"] * m["vdim"]
+            n += 2 * W + W * cfg.canon_taps + W * W + W
+            if l.mlp:
+                n += l.mlp["router"]["experts"] * 3 * W * l.mlp["expert"]["ff"] + 2 * W + W * W + W
+        return n
     if isinstance(cfg, PemidraConfig):
         W, n = cfg.hidden, 2 * cfg.vocab_size * cfg.hidden + 2 * cfg.hidden
         for l in cfg.layers:

@@ -19,7 +19,8 @@ from .mixers import (conv_silu, embed_pos, gated_group_rmsnorm, linear_swiglu_an
                      sig_prefill_tiles, sigattn_supported, sigmoid_attention_decode, sigmoid_attention_prefill,
                      softcap, ssm_scan, stream_rmsnorm, unitnorm_kv_write, embed_stream, stream_layernorm, gelu_tanh_mul,
                      dual_rmsnorm_mean, normrope_kv_write, sink_attention_prefill, sink_attention_decode, mask_first_key,
-                     MASK_CAUSAL, MASK_CHUNK, MASK_WINDOW)
+                     pooled_blocks_seen, MASK_CAUSAL, MASK_CHUNK, MASK_WINDOW)
+from .window import moe_route, pool_kv_write, rms_cols, rot_kv_write, stream_gated_norm, table_experts  # noqa: F401
 from .delta import (delta_scan, delta_scan_supported, gated_delta_prep, general_delta_prep, head_norm_gate, tanh_,  # noqa: F401
                     GATE_SIGMOID, GATE_SILU)
 

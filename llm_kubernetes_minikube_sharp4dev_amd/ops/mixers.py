@@ -25,7 +25,8 @@ from ._ext import lib, use_hip
 __all__ = ["embed_pos", "stream_rmsnorm", "softcap", "linear_swiglu_any", "unitnorm_kv_write", "sig_prefill_tiles", "sig_decode_splits",
            "sigmoid_attention_prefill", "sigmoid_attention_decode", "sigattn_supported", "conv_silu", "ssm_scan",
            "gated_group_rmsnorm", "embed_stream", "stream_layernorm", "gelu_tanh_mul", "dual_rmsnorm_mean", "normrope_kv_write",
-           "sink_attention_prefill", "sink_attention_decode", "mask_first_key", "MASK_CAUSAL", "MASK_CHUNK", "MASK_WINDOW"]
+           "sink_attention_prefill", "sink_attention_decode", "mask_first_key", "pooled_blocks_seen", "MASK_CAUSAL", "MASK_CHUNK",
+           "MASK_WINDOW"]
 
 SIG_TILE_ROWS = 16       # queries per wave of the prefill kernel
 SIG_MAX_HEAD = 256       # largest per-head q/k or v size the kernels are built for
@@ -205,12 +206,13 @@ def sigmoid_attention_decode(q, k_cache, v_cache, block_tables, ctx_lens, H: int
 
 
 # ------------------------------------------------------------------ state-space mixer
-def conv_silu(u, col0: int, C: int, w, bias, state, cu, slots, positions, max_len: int):
+def conv_silu(u, col0: int, C: int, w, bias, state, cu, slots, positions, max_len: int, act: bool = True):
     """silu(causal depthwise conv + bias) of columns [col0, col0 + C) of ``u``, per sequence, reading
     the inputs before a chunk from ``state`` and leaving the sequence's last ``taps - 1`` inputs there.
-    w f32 [C, taps] (last column = the current token), bias f32 [C] or None."""
+    w f32 [C, taps] (last column = the current token), bias f32 [C] or None.  ``act`` False: the
+    convolution alone, without the SiLU."""
     if use_hip(u):
-        return lib().conv_silu(u, col0, C, w, bias, state, cu, slots, positions, int(max_len))
+        return lib().conv_silu(u, col0, C, w, bias, state, cu, slots, positions, int(max_len), bool(act))
     taps = w.shape[1]
     out = torch.zeros(u.shape[0], C, dtype=u.dtype, device=u.device)
     cul, sl = cu.tolist(), slots.tolist()
@@ -231,7 +233,7 @@ def conv_silu(u, col0: int, C: int, w, bias, state, cu, slots, positions, max_le
             acc += ff[k:k + r1 - r0] * w[:, k]
         if bias is not None:
             acc += bias
-        out[r0:r1] = F.silu(acc).to(u.dtype)
+        out[r0:r1] = (F.silu(acc) if act else acc).to(u.dtype)
     return out
 
 
@@ -279,13 +281,15 @@ def gated_group_rmsnorm(y, z, w, ngroups: int, eps: float):
 
 
 # ------------------------------------------------------------------ post-norm f32 stream
-def embed_stream(ids, tok, out_dtype=torch.bfloat16):
-    """(x f32 [T, W], h): the token rows as the f32 stream and as the activation-dtype copy the
-    projections read (for f32 activations both are the same tensor)."""
+def embed_stream(ids, tok, out_dtype=torch.bfloat16, scale: float = 1.0):
+    """(x f32 [T, W], h): the token rows times ``scale`` (an f32 product) as the f32 stream and as the
+    activation-dtype copy the projections read (for f32 activations both are the same tensor)."""
     if use_hip(tok):
-        x, h = lib().embed_stream(ids, tok, out_dtype)
+        x, h = lib().embed_stream(ids, tok, out_dtype, float(scale))
         return x, h
     x = tok[ids.long()].float()
+    if scale != 1.0:
+        x = x * scale
     return x, (x if out_dtype == torch.float32 else x.to(out_dtype))
 
 
@@ -385,13 +389,38 @@ def normrope_kv_write(qkv, H: int, G: int, dim: int, vdim: int, q_w, k_w, rot_di
     return qkv
 
 
-def _sink_rows(q, k, v, qpos, hscale, mask_kind, mask_size, sink):
-    """q f32 [S, H, dim] at positions qpos [S]; k/v f32 [n, G, *] at positions 0..n-1."""
+def pooled_blocks_seen(qpos, mask_size: int, pool: int):
+    """Number of leading blocks of ``pool`` positions that the window of ``mask_size`` positions ending at
+    ``qpos`` has left behind entirely (block b is seen when b * pool + pool - 1 <= qpos - mask_size)."""
+    if isinstance(qpos, torch.Tensor):
+        return ((qpos - mask_size + 1).clamp(min=0)) // pool
+    return max(0, qpos - mask_size + 1) // pool
+
+
+def _sink_rows(q, k, v, qpos, hscale, mask_kind, mask_size, sink, pooled=None):
+    """q f32 [S, H, dim] at positions qpos [S]; k/v f32 [n, G, *] at positions 0..n-1.  ``pooled`` = (pk, pv
+    f32 [nb, G, *], pool): one more key / value per block of ``pool`` positions, seen by a query once the
+    block is entirely behind its window, in the same softmax."""
     H, G = q.shape[1], k.shape[1]
     rep = H // G
     s = torch.einsum("ihd,jhd->hij", q, k.repeat_interleave(rep, dim=1)) * hscale.view(-1, 1, 1)
     j = torch.arange(k.shape[0], device=q.device).view(1, -1)
     i = qpos.view(-1, 1)
+    if pooled is not None and pooled[0].shape[0]:
+        pk, pv, pool = pooled
+        sp = torch.einsum("ihd,jhd->hij", q, pk.repeat_interleave(rep, dim=1)) * hscale.view(-1, 1, 1)
+        bj = torch.arange(pk.shape[0], device=q.device).view(1, -1)
+        sp = sp.masked_fill(~(bj < pooled_blocks_seen(i, mask_size, pool))[None], float("-inf"))
+        lo = (i - mask_size + 1).clamp(min=0)
+        s = s.masked_fill(~((j <= i) & (j >= lo))[None], float("-inf"))
+        s = torch.cat([sp, s], -1)
+        m = s.amax(-1, keepdim=True)
+        if sink:
+            m = m.clamp(min=0.0)
+        e = torch.exp(s - m)
+        den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sink else 0.0)
+        vv = torch.cat([pv, v], 0).repeat_interleave(rep, dim=1)
+        return torch.einsum("hij,jhd->ihd", e / den, vv)
     if mask_kind == MASK_CHUNK:
         lo = (i // mask_size) * mask_size
     elif mask_kind == MASK_WINDOW:
@@ -400,26 +429,48 @@ def _sink_rows(q, k, v, qpos, hscale, mask_kind, mask_size, sink):
         lo = torch.zeros_like(i)
     seen = (j <= i) & (j >= lo)
     s = s.masked_fill(~seen[None], float("-inf"))
-    m = s.amax(-1, keepdim=True).clamp(min=0.0)          # the sink's score 0 bounds the maximum from below
+    m = s.amax(-1, keepdim=True)
+    if sink:
+        m = m.clamp(min=0.0)                             # the sink's score 0 bounds the maximum from below
     e = torch.exp(s - m)
     den = e.sum(-1, keepdim=True) + (torch.exp(-m) if sink else 0.0)
     return torch.einsum("hij,jhd->ihd", e / den, v.repeat_interleave(rep, dim=1))
 
 
+def _pooled_of(pool, table, n):
+    """(pk, pv f32 [n // P, G, *], P) of a sequence of ``n`` cached tokens: pooled entry b lives at the
+    logical position b of the sequence's own block table in the pooled cache pair."""
+    if pool is None:
+        return None
+    pk_cache, pv_cache, P = pool
+    nb = n // P
+    if nb == 0:
+        return (torch.zeros(0, pk_cache.shape[1], pk_cache.shape[3]), torch.zeros(0, pv_cache.shape[1], pv_cache.shape[2]), P)
+    pk, pv = _gather_kv(pk_cache, pv_cache, table, nb)
+    return pk, pv, P
+
+
 def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H: int, G: int, dim: int, vdim: int, hscale,
-                           mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, tiles=None, q_lens_cpu=None):
+                           mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, tiles=None, q_lens_cpu=None,
+                           pool=None):
     """Softmax attention of query chunks over their sequences' cached keys inside the mask
     (``mask_first_key``), with ``sink``: one more term of score 0 and no value in the denominator.
     ``hscale`` f32 [H]: the score multiplier of each head.  ``gate`` (or None): rows aligned with ``q``
     whose columns ``gate_col + h`` hold the raw output gate of head h; the head's output is multiplied by
-    its sigmoid.  q: rows whose first H * dim columns are the prepared queries; out [T, H * vdim]."""
+    its sigmoid.  q: rows whose first H * dim columns are the prepared queries; out [T, H * vdim].
+    ``pool`` = (pooled K cache, pooled V cache, P), window masks only: beside its window a query sees one
+    pooled key / value per block of P positions entirely behind the window (``pooled_blocks_seen``), filed by
+    ``pool_kv_write`` at the logical position b of the same block table."""
+    if pool is not None and mask_kind != MASK_WINDOW:
+        raise ValueError("pooled blocks go with a sliding window")
     if use_hip(q):
         if tiles is None:
             ql = q_lens_cpu if q_lens_cpu is not None else (cu_q[1:] - cu_q[:-1]).tolist()
             ts, tq = sig_prefill_tiles(ql, ctx_lens.tolist())
             tiles = (torch.from_numpy(ts).to(q.device), torch.from_numpy(tq).to(q.device))
+        pk, pv, P = pool if pool is not None else (None, None, 0)
         lib().sinkattn_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, tiles[0], tiles[1], H, G, dim, vdim, hscale,
-                               int(mask_kind), int(mask_size), bool(sink), gate, int(gate_col), out)
+                               int(mask_kind), int(mask_size), bool(sink), gate, int(gate_col), out, pk, pv, int(P))
         return out
     cu = cu_q.tolist()
     for b in range(len(cu) - 1):
@@ -428,7 +479,7 @@ def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H:
         k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
         qq = q[s0:s1, : H * dim].float().view(s1 - s0, H, dim)
         qpos = torch.arange(n - (s1 - s0), n, device=q.device)
-        o = _sink_rows(qq, k, v, qpos, hscale, mask_kind, mask_size, sink)
+        o = _sink_rows(qq, k, v, qpos, hscale, mask_kind, mask_size, sink, _pooled_of(pool, block_tables[b], n))
         if gate is not None:
             o = o * torch.sigmoid(gate[s0:s1, gate_col:gate_col + H].float()).unsqueeze(-1)
         out[s0:s1, : H * vdim] = o.reshape(s1 - s0, H * vdim).to(out.dtype)
@@ -436,20 +487,26 @@ def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H:
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, ctx_lens, H: int, G: int, dim: int, vdim: int, hscale,
-                          mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, splits: int = 1, part=None):
-    """One query row per sequence at its last position (ctx - 1) over its cached keys inside the mask."""
+                          mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, splits: int = 1, part=None,
+                          pool=None):
+    """One query row per sequence at its last position (ctx - 1) over its cached keys inside the mask
+    (and the pooled blocks before it: see ``sink_attention_prefill``)."""
     B = q.shape[0]
+    if pool is not None and mask_kind != MASK_WINDOW:
+        raise ValueError("pooled blocks go with a sliding window")
     if use_hip(q):
         if splits > 1 and part is None:
             part = torch.empty(B * H * splits * (vdim + 2), dtype=torch.float32, device=q.device)
+        pk, pv, P = pool if pool is not None else (None, None, 0)
         lib().sinkattn_decode(q, k_cache, v_cache, block_tables, ctx_lens, int(splits), H, G, dim, vdim, hscale, int(mask_kind),
-                              int(mask_size), bool(sink), gate, int(gate_col), out, part)
+                              int(mask_size), bool(sink), gate, int(gate_col), out, part, pk, pv, int(P))
         return out
     for b in range(B):
         n = int(ctx_lens[b])
         k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
         qq = q[b:b + 1, : H * dim].float().view(1, H, dim)
-        o = _sink_rows(qq, k, v, torch.tensor([n - 1], device=q.device), hscale, mask_kind, mask_size, sink)
+        o = _sink_rows(qq, k, v, torch.tensor([n - 1], device=q.device), hscale, mask_kind, mask_size, sink,
+                       _pooled_of(pool, block_tables[b], n))
         if gate is not None:
             o = o * torch.sigmoid(gate[b:b + 1, gate_col:gate_col + H].float()).unsqueeze(-1)
         out[b:b + 1, : H * vdim] = o.reshape(1, H * vdim).to(out.dtype)
