@@ -9,6 +9,12 @@
 // portions, a decode row and a whole prompt give the same sums; keys outside the mask are never read
 // beyond the 32-key step that holds the first visible one.
 //
+// Pooled blocks (window masks, pool > 0): beside its window a query sees one more key / value per block of
+// `pool` positions that the window has left behind entirely -- block b once b * pool + pool - 1 <= i - msize, i.e.
+// the first max(0, i - msize + 1) / pool blocks -- in the same softmax.  The pooled keys and values live in a
+// second cache pair of the same layout, entry b at the logical position b of the sequence's block table, so
+// the pass over them is the pass over the window with other pointers and the bound "b < blocks seen".
+//
 // lk_normrope_kv_write prepares the operands in f32: q and k RMS-normed per head with a weight shared by
 // the heads, their first `rot` dimensions rotated by the position (dimension i pairs with i + rot / 2),
 // v divided by its RMS; q in place, k and v into the cache.
@@ -44,7 +50,19 @@ struct SinkParams {
   const void* gate;     // rows aligned with q; column gcol + h (null: no gate)
   long gs;
   int gcol;
+  const void* pkc;      // pooled K / V caches (pool > 0)
+  const void* pvc;
+  int pool;
 };
+
+LK_DEVICE int blocks_seen(int qpos, int msize, int pool) { return max(0, qpos - msize + 1) / pool; }
+
+LK_DEVICE SinkParams pooled_view(const SinkParams& p) {
+  SinkParams r = p;
+  r.kc = p.pkc;
+  r.vc = p.pvc;
+  return r;
+}
 
 LK_DEVICE int first_key(int qpos, int mkind, int msize) {
   if (mkind == 1) return (qpos / msize) * msize;
@@ -256,6 +274,12 @@ __global__ __launch_bounds__(256) void sinkattn_prefill_kernel(SinkParams p, con
   const int k0 = first_key(past + q0, p.mkind, p.msize) & ~31;   // first(i) never decreases with i
   sink_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, k0, k1, WT ? 0 : w, WT ? 1 : 4, cvalid, qpos,
                    first_key(qpos, p.mkind, p.msize), p.hscale[head], m, l, o);
+  if (p.pool > 0) {
+    const int nbt = blocks_seen(k1 - 1, p.msize, p.pool);   // the tile's last query sees the most blocks
+    if (nbt > 0)
+      sink_run<T, PAD>(pooled_view(p), qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, nbt, WT ? 0 : w, WT ? 1 : 4,
+                       cvalid, blocks_seen(qpos, p.msize, p.pool) - 1, 0, p.hscale[head], m, l, o);
+  }
   if constexpr (WT) {
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -300,11 +324,16 @@ __global__ __launch_bounds__(256) void sinkattn_decode_kernel(SinkParams p, cons
   for (int vt = 0; vt < VT; ++vt) o[vt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m = p.sink ? 0.f : kNegBig, l = 0.f;
   const int klo = first_key(ctx - 1, p.mkind, p.msize), k0 = klo & ~31;
-  const int nsteps = (ctx - k0 + 31) / 32, spz = (nsteps + Z - 1) / Z;
+  // the key splits share the window's 32-key steps and, behind them, the steps over the pooled blocks
+  const int nb = p.pool > 0 ? blocks_seen(ctx - 1, p.msize, p.pool) : 0;
+  const int nwin = (ctx - k0 + 31) / 32, nsteps = nwin + (nb + 31) / 32, spz = (nsteps + Z - 1) / Z;
   const int s0 = z * spz, s1 = min(nsteps, s0 + spz);
-  if (s0 < s1)
-    sink_run<T, PAD>(p, qf, kvh, p.bt + (long)b * p.bt_stride, k0 + 32 * s0, min(ctx, k0 + 32 * s1), w, 4, cvalid, ctx - 1, klo,
-                     p.hscale[head], m, l, o);
+  if (s0 < min(s1, nwin))
+    sink_run<T, PAD>(p, qf, kvh, p.bt + (long)b * p.bt_stride, k0 + 32 * s0, min(ctx, k0 + 32 * min(s1, nwin)), w, 4, cvalid, ctx - 1,
+                     klo, p.hscale[head], m, l, o);
+  if (max(s0, nwin) < s1)
+    sink_run<T, PAD>(pooled_view(p), qf, kvh, p.bt + (long)b * p.bt_stride, 32 * (max(s0, nwin) - nwin), min(nb, 32 * (s1 - nwin)), w, 4,
+                     cvalid, nb - 1, 0, p.hscale[head], m, l, o);
   merge_waves<EXACT, VT>(m, l, o, red, ml);
   if (w == 0 && cvalid) {
     if (Z == 1) {
@@ -440,7 +469,8 @@ int pad_of(int dim, int vdim) {
 bool shape_ok(const SinkParams& p, int esz) {
   const int ev = 16 / esz;
   return p.H > 0 && p.G > 0 && p.H % p.G == 0 && p.dim > 0 && p.vdim > 0 && p.dim % ev == 0 && p.vdim % ev == 0 && p.BS % 16 == 0 &&
-         pad_of(p.dim, p.vdim) != 0 && p.mkind >= 0 && p.mkind <= 2 && (p.mkind == 0 || p.msize >= 1);
+         pad_of(p.dim, p.vdim) != 0 && p.mkind >= 0 && p.mkind <= 2 && (p.mkind == 0 || p.msize >= 1) && p.pool >= 0 &&
+         (p.pool == 0 || (p.mkind == 2 && p.pkc != nullptr && p.pvc != nullptr));
 }
 
 template <typename T, int PAD>
@@ -490,11 +520,12 @@ int decode_t(const SinkParams& p, const int* ctx, int B, int Z, void* out, long 
 }
 
 SinkParams make_params(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, int H, int G, int dim,
-                       int vdim, int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol) {
+                       int vdim, int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol,
+                       const void* pkc, const void* pvc, int pool) {
   SinkParams p;
   p.q = q; p.qs = qs; p.kc = kc; p.vc = vc; p.bt = bt; p.bt_stride = bt_stride;
   p.H = H; p.G = G; p.dim = dim; p.vdim = vdim; p.BS = BS; p.hscale = hscale; p.mkind = mkind; p.msize = msize; p.sink = sink;
-  p.gate = gate; p.gs = gs; p.gcol = gcol;
+  p.gate = gate; p.gs = gs; p.gcol = gcol; p.pkc = pkc; p.pvc = pvc; p.pool = pool;
   return p;
 }
 
@@ -520,9 +551,9 @@ int lk_normrope_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int 
 int lk_sinkattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* cu_q,
                         const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H, int G, int dim, int vdim,
                         int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol, void* out,
-                        long os, int esz, hipStream_t st) {
+                        long os, const void* pkc, const void* pvc, int pool, int esz, hipStream_t st) {
   if (ntiles <= 0) return 0;
-  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol);
+  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol, pkc, pvc, pool);
   if (!shape_ok(p, esz)) return -1;
   return esz == 2 ? prefill_t<bf16_t>(p, cu_q, ctx_lens, tile_seq, tile_q0, ntiles, out, os, st)
                   : prefill_t<float>(p, cu_q, ctx_lens, tile_seq, tile_q0, ntiles, out, os, st);
@@ -530,9 +561,10 @@ int lk_sinkattn_prefill(const void* q, long qs, const void* kc, const void* vc, 
 
 int lk_sinkattn_decode(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* ctx_lens,
                        int B, int Z, int H, int G, int dim, int vdim, int BS, const float* hscale, int mkind, int msize, int sink,
-                       const void* gate, long gs, int gcol, void* out, long os, float* part, int esz, hipStream_t st) {
+                       const void* gate, long gs, int gcol, void* out, long os, float* part, const void* pkc, const void* pvc,
+                       int pool, int esz, hipStream_t st) {
   if (B <= 0) return 0;
-  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol);
+  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol, pkc, pvc, pool);
   if (!shape_ok(p, esz) || Z < 1 || (Z > 1 && part == nullptr)) return -1;
   return esz == 2 ? decode_t<bf16_t>(p, ctx_lens, B, Z, out, os, part, st) : decode_t<float>(p, ctx_lens, B, Z, out, os, part, st);
 }

@@ -1219,7 +1219,7 @@ void check_seqs(const at::Tensor& cu, const at::Tensor& slots, const at::Tensor&
 // u: [T, >= col0 + C] rows of the input projection; the convolved channels are columns [col0, col0 + C)
 at::Tensor conv_silu(const at::Tensor& u, int64_t col0, int64_t C, const at::Tensor& w, const c10::optional<at::Tensor>& bias,
                      at::Tensor& state, const at::Tensor& cu, const at::Tensor& slots, const at::Tensor& positions,
-                     int64_t max_len) {
+                     int64_t max_len, bool act) {
   CHECK_CUDA(u); CHECK_LASTDIM(u);
   const int esz = esz_of(u, "u");
   TORCH_CHECK(u.dim() == 2 && col0 >= 0 && col0 + C <= u.size(1), "u columns");
@@ -1232,7 +1232,7 @@ at::Tensor conv_silu(const at::Tensor& u, int64_t col0, int64_t C, const at::Ten
   at::Tensor out = at::empty({u.size(0), C}, u.options());
   CHECK_RC(lk_conv_silu((const char*)u.data_ptr() + col0 * esz, u.stride(0), C, taps, fp(w, C * taps, "conv weight"),
                         fpo(bias, C, "conv bias"), state.data_ptr(), ip(cu), ip(slots), ip(positions), cu.numel() - 1, max_len,
-                        out.data_ptr(), out.stride(0), esz, cur_stream()), "conv_silu");
+                        out.data_ptr(), out.stride(0), act ? 1 : 0, esz, cur_stream()), "conv_silu");
   return out;
 }
 
@@ -1268,7 +1268,7 @@ at::Tensor gated_group_rmsnorm(const at::Tensor& y, const at::Tensor& z, const a
 
 // ---------------------------------------------------------------------------------------------
 // post-norm f32 stream, linear-state scans, softmax attention with a sink (bf16 or f32 activations)
-std::vector<at::Tensor> embed_stream(const at::Tensor& ids, const at::Tensor& tok, at::ScalarType out_dtype) {
+std::vector<at::Tensor> embed_stream(const at::Tensor& ids, const at::Tensor& tok, at::ScalarType out_dtype, double scale) {
   CHECK_CUDA(ids); CHECK_I32(ids); CHECK_CONTIG(ids); CHECK_CUDA(tok); CHECK_CONTIG(tok);
   const int esz = esz_of(tok, "tok");
   TORCH_CHECK(tok.dim() == 2 && tok.scalar_type() == out_dtype, "token table must be [V, W] in the activation dtype");
@@ -1276,7 +1276,7 @@ std::vector<at::Tensor> embed_stream(const at::Tensor& ids, const at::Tensor& to
   const int W = tok.size(1);
   at::Tensor x = at::empty({T, W}, tok.options().dtype(at::kFloat));
   at::Tensor copy = esz == 2 ? at::empty({T, W}, tok.options()) : x;
-  CHECK_RC(lk_embed_stream(ip(ids), tok.data_ptr(), tok.size(0), T, W, x.data_ptr<float>(), esz == 2 ? copy.data_ptr() : nullptr, esz,
+  CHECK_RC(lk_embed_stream(ip(ids), tok.data_ptr(), tok.size(0), T, W, x.data_ptr<float>(), esz == 2 ? copy.data_ptr() : nullptr, (float)scale, esz,
                            cur_stream()), "embed_stream");
   return {x, copy};
 }
@@ -1453,12 +1453,27 @@ const void* gate_rows(const c10::optional<at::Tensor>& gate, const at::Tensor& q
   return gate->data_ptr();
 }
 
+// the pooled cache pair of a window mask (pool > 0): the same shapes and type as the K / V caches
+void pooled_caches(const at::Tensor& q, const at::Tensor& kc, const c10::optional<at::Tensor>& pkc, const c10::optional<at::Tensor>& pvc,
+                   int64_t pool, int64_t G, int64_t dim, int64_t vdim, const void** pkp, const void** pvp) {
+  TORCH_CHECK(pool >= 0, "pool");
+  if (pool == 0) return;
+  TORCH_CHECK(pkc.has_value() && pvc.has_value(), "pooled caches are missing");
+  check_sig_caches(q, *pkc, *pvc, G, dim, vdim);
+  TORCH_CHECK(pkc->size(0) == kc.size(0) && pkc->size(2) == kc.size(2), "pooled caches must have the K / V caches' blocks");
+  *pkp = pkc->data_ptr();
+  *pvp = pvc->data_ptr();
+}
+
 void sinkattn_prefill(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt, const at::Tensor& cu_q,
                       const at::Tensor& ctx, const at::Tensor& tile_seq, const at::Tensor& tile_q0, int64_t H, int64_t G, int64_t dim,
                       int64_t vdim, const at::Tensor& hscale, int64_t mkind, int64_t msize, bool sink,
-                      const c10::optional<at::Tensor>& gate, int64_t gate_col, at::Tensor& out) {
+                      const c10::optional<at::Tensor>& gate, int64_t gate_col, at::Tensor& out,
+                      const c10::optional<at::Tensor>& pkc, const c10::optional<at::Tensor>& pvc, int64_t pool) {
   CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(out); CHECK_LASTDIM(out);
   const int esz = esz_of(q, "q");
+  const void *pkp = nullptr, *pvp = nullptr;
+  pooled_caches(q, kc, pkc, pvc, pool, G, dim, vdim, &pkp, &pvp);
   same_type(out, q, "out");
   TORCH_CHECK(q.dim() == 2 && q.size(1) >= H * dim && out.dim() == 2 && out.size(0) == q.size(0) && out.size(1) >= H * vdim, "q / out shape");
   check_rows16(q, "q");
@@ -1472,15 +1487,18 @@ void sinkattn_prefill(const at::Tensor& q, const at::Tensor& kc, const at::Tenso
   CHECK_RC(lk_sinkattn_prefill(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), (int)bt.stride(0), ip(cu_q), ip(ctx),
                                ip(tile_seq), ip(tile_q0), (int)tile_seq.numel(), (int)H, (int)G, (int)dim, (int)vdim, (int)kc.size(2),
                                fp(hscale, H, "hscale"), (int)mkind, (int)msize, sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(),
-                               out.stride(0), esz, cur_stream()), "sinkattn_prefill");
+                               out.stride(0), pkp, pvp, (int)pool, esz, cur_stream()), "sinkattn_prefill");
 }
 
 void sinkattn_decode(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt, const at::Tensor& ctx,
                      int64_t Z, int64_t H, int64_t G, int64_t dim, int64_t vdim, const at::Tensor& hscale, int64_t mkind,
                      int64_t msize, bool sink, const c10::optional<at::Tensor>& gate, int64_t gate_col, at::Tensor& out,
-                     const c10::optional<at::Tensor>& part) {
+                     const c10::optional<at::Tensor>& part, const c10::optional<at::Tensor>& pkc,
+                     const c10::optional<at::Tensor>& pvc, int64_t pool) {
   CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(out); CHECK_LASTDIM(out);
   const int esz = esz_of(q, "q");
+  const void *pkp = nullptr, *pvp = nullptr;
+  pooled_caches(q, kc, pkc, pvc, pool, G, dim, vdim, &pkp, &pvp);
   same_type(out, q, "out");
   const long B = q.size(0);
   TORCH_CHECK(q.dim() == 2 && q.size(1) >= H * dim && out.dim() == 2 && out.size(0) == B && out.size(1) >= H * vdim, "q / out shape");
@@ -1498,8 +1516,138 @@ void sinkattn_decode(const at::Tensor& q, const at::Tensor& kc, const at::Tensor
   const void* gp = gate_rows(gate, q, gate_col, H, &gs);
   CHECK_RC(lk_sinkattn_decode(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), (int)bt.stride(0), ip(ctx), (int)B, (int)Z,
                               (int)H, (int)G, (int)dim, (int)vdim, (int)kc.size(2), fp(hscale, H, "hscale"), (int)mkind, (int)msize,
-                              sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(), out.stride(0), pp, esz, cur_stream()),
+                              sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(), out.stride(0), pp, pkp, pvp, (int)pool, esz,
+                              cur_stream()),
            "sinkattn_decode");
+}
+
+// ---------------------------------------------------------------------------------------------
+// windowed attention with pooled blocks, latent attention, table-routed experts
+c10::optional<at::Tensor> stream_gated_norm(at::Tensor& x, const at::Tensor& y, int64_t parts, const at::Tensor& g, const at::Tensor& gb,
+                                            const at::Tensor& wpost, const c10::optional<at::Tensor>& wnext, double eps,
+                                            at::ScalarType out_dtype) {
+  CHECK_CUDA(x); CHECK_F32(x); CHECK_CONTIG(x); CHECK_CUDA(y); CHECK_LASTDIM(y); CHECK_CUDA(g); CHECK_LASTDIM(g);
+  const int esz = esz_of(y, "y");
+  same_type(g, y, "g");
+  TORCH_CHECK(x.dim() == 2 && y.dim() == 2 && g.dim() == 2 && parts >= 1, "x, y, g must be 2-d");
+  const long T = x.size(0);
+  const int W = x.size(1);
+  TORCH_CHECK(y.size(0) == T * parts && y.size(1) == W && g.size(0) == T && g.size(1) == W, "y must be [T * parts, W], g [T, W]");
+  TORCH_CHECK(y.scalar_type() == out_dtype, "out dtype must be the activations'");
+  at::Tensor out;
+  if (wnext) out = at::empty({T, W}, y.options());
+  CHECK_RC(lk_stream_gated_norm(x.data_ptr<float>(), y.data_ptr(), y.stride(0), (int)parts, g.data_ptr(), g.stride(0), fp(gb, W, "gate bias"),
+                                fp(wpost, W, "post norm weight"), fpo(wnext, W, "next norm weight"), (float)eps,
+                                wnext ? out.data_ptr() : nullptr, wnext ? out.stride(0) : 0, T, W, esz, cur_stream()),
+           "stream_gated_norm");
+  if (!wnext) return c10::nullopt;
+  return out;
+}
+
+at::Tensor rms_cols(const at::Tensor& u, int64_t col0, int64_t n, const at::Tensor& w, double eps) {
+  CHECK_CUDA(u); CHECK_LASTDIM(u);
+  const int esz = esz_of(u, "u");
+  TORCH_CHECK(u.dim() == 2 && col0 >= 0 && n >= 1 && col0 + n <= u.size(1), "u columns");
+  at::Tensor out = at::empty({u.size(0), n}, u.options());
+  CHECK_RC(lk_rms_cols((const char*)u.data_ptr() + col0 * esz, u.stride(0), (int)n, fp(w, n, "norm weight"), (float)eps, out.data_ptr(),
+                       out.stride(0), u.size(0), esz, cur_stream()), "rms_cols");
+  return out;
+}
+
+void rot_kv_write(at::Tensor& q, int64_t H, int64_t qdim, const at::Tensor& k, int64_t G, int64_t kdim,
+                  const c10::optional<at::Tensor>& kshared, int64_t sdim, const at::Tensor& v, int64_t vdim, int64_t rot_off,
+                  int64_t rot, const at::Tensor& freq, double mag, const at::Tensor& positions, at::Tensor& kc, at::Tensor& vc,
+                  const at::Tensor& slots) {
+  CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(k); CHECK_LASTDIM(k); CHECK_CUDA(v); CHECK_LASTDIM(v);
+  CHECK_CUDA(slots); CHECK_I32(slots); CHECK_CONTIG(slots); CHECK_CUDA(positions); CHECK_I32(positions); CHECK_CONTIG(positions);
+  const int esz = esz_of(q, "q");
+  same_type(k, q, "k"); same_type(v, q, "v");
+  const long T = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && k.dim() == 2 && v.dim() == 2 && k.size(0) == T && v.size(0) == T, "q, k, v rows");
+  TORCH_CHECK(H >= 1 && G >= 1 && q.size(1) >= H * qdim && k.size(1) >= G * kdim && v.size(1) >= G * vdim, "q, k, v columns");
+  TORCH_CHECK(slots.numel() >= T && positions.numel() >= T, "slots / positions");
+  const void* shp = nullptr;
+  long shs = 0;
+  if (sdim > 0) {
+    TORCH_CHECK(kshared.has_value(), "shared key part is missing");
+    CHECK_CUDA(*kshared); CHECK_LASTDIM(*kshared); same_type(*kshared, q, "kshared");
+    TORCH_CHECK(kshared->dim() == 2 && kshared->size(0) == T && kshared->size(1) >= sdim, "shared key part must be [T, >= sdim]");
+    shp = kshared->data_ptr();
+    shs = kshared->stride(0);
+  }
+  CHECK_CUDA(kc); CHECK_CUDA(vc); CHECK_CONTIG(kc); CHECK_CONTIG(vc); same_type(kc, q, "k cache"); same_type(vc, q, "v cache");
+  TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.size(1) == G && vc.size(1) == G && kc.size(0) == vc.size(0) && vc.size(3) == kc.size(2),
+              "caches must be K [NB, G, BS, KD], V [NB, G, VD, BS]");
+  CHECK_CUDA(freq); CHECK_F32(freq); CHECK_CONTIG(freq);
+  TORCH_CHECK(rot >= 0 && rot % 2 == 0 && freq.numel() >= rot / 2, "rot / freq");
+  CHECK_RC(lk_rot_kv_write(q.data_ptr(), q.stride(0), (int)H, (int)qdim, k.data_ptr(), k.stride(0), (int)G, (int)kdim, shp, shs, (int)sdim,
+                           v.data_ptr(), v.stride(0), (int)vdim, (int)rot_off, (int)rot, freq.data_ptr<float>(), (float)mag,
+                           ip(positions), kc.data_ptr(), vc.data_ptr(), ip(slots), (int)kc.size(2), (int)kc.size(3), (int)vc.size(2), T,
+                           esz, cur_stream()), "rot_kv_write");
+}
+
+void pool_kv_write(const at::Tensor& kc, const at::Tensor& vc, at::Tensor& pkc, at::Tensor& pvc, int64_t P, const at::Tensor& bt,
+                   const at::Tensor& ctx, const c10::optional<at::Tensor>& cu_q, const at::Tensor& slots, int64_t row0,
+                   int64_t max_len) {
+  CHECK_CUDA(kc); CHECK_CUDA(vc); CHECK_CUDA(pkc); CHECK_CUDA(pvc); CHECK_CONTIG(kc); CHECK_CONTIG(vc); CHECK_CONTIG(pkc); CHECK_CONTIG(pvc);
+  const int esz = esz_of(kc, "k cache");
+  same_type(vc, kc, "v cache"); same_type(pkc, kc, "pooled k cache"); same_type(pvc, kc, "pooled v cache");
+  TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.sizes() == pkc.sizes() && vc.sizes() == pvc.sizes() && kc.size(0) == vc.size(0) &&
+              kc.size(1) == vc.size(1) && vc.size(3) == kc.size(2), "caches must be K [NB, G, BS, dim], V [NB, G, vdim, BS], pooled pair alike");
+  CHECK_CUDA(bt); CHECK_I32(bt); CHECK_CUDA(ctx); CHECK_I32(ctx); CHECK_CONTIG(ctx); CHECK_CUDA(slots); CHECK_I32(slots); CHECK_CONTIG(slots);
+  const long S = cu_q ? cu_q->numel() - 1 : ctx.numel();
+  if (cu_q) { CHECK_CUDA(*cu_q); CHECK_I32(*cu_q); CHECK_CONTIG(*cu_q); }
+  TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1 && bt.size(0) >= S && ctx.numel() >= S && P >= 1 && row0 >= 0 && max_len >= 1,
+              "block tables / lengths");
+  TORCH_CHECK(cu_q.has_value() || slots.numel() >= row0 + S, "slots");
+  CHECK_RC(lk_pool_kv_write(kc.data_ptr(), vc.data_ptr(), pkc.data_ptr(), pvc.data_ptr(), (int)P, ip(bt), (int)bt.stride(0), ip(ctx),
+                            ipo(cu_q), ip(slots), (int)row0, (int)S, (int)max_len, (int)kc.size(1), (int)kc.size(2), (int)kc.size(3),
+                            (int)vc.size(2), esz, cur_stream()), "pool_kv_write");
+}
+
+// x [rows, K] sorted by expert -- or, with `gather` int32 [rows], any x whose row gather[r] is sorted row r's input; the
+// result's rows are sorted, or with `scatter` int32 [rows] sorted row r lands in out row scatter[r] (a permutation)
+at::Tensor gemm_grouped(const at::Tensor& x, const at::Tensor& seg, const at::Tensor& w, bool swiglu,
+                        const c10::optional<at::Tensor>& gather, const c10::optional<at::Tensor>& scatter) {
+  CHECK_CUDA(x); CHECK_BF16(x); CHECK_LASTDIM(x); CHECK_CUDA(w); CHECK_BF16(w); CHECK_CONTIG(w); CHECK_CUDA(seg); CHECK_I32(seg);
+  CHECK_CONTIG(seg);
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 3 && w.size(2) == x.size(1) && seg.numel() == w.size(0) + 1, "x [rows, K], w [E, N, K], seg [E + 1]");
+  const int N = w.size(1), K = w.size(2);
+  TORCH_CHECK(lk_gemm_grouped_supported(N, K, swiglu ? 1 : 0), "shape not tiled by the grouped GEMM");
+  long rows = x.size(0);
+  if (gather) { CHECK_CUDA(*gather); CHECK_I32(*gather); CHECK_CONTIG(*gather); rows = gather->numel(); }
+  if (scatter) { CHECK_CUDA(*scatter); CHECK_I32(*scatter); CHECK_CONTIG(*scatter); TORCH_CHECK(scatter->numel() == rows, "scatter rows"); }
+  at::Tensor out = at::empty({rows, swiglu ? N / 2 : N}, x.options());
+  CHECK_RC(lk_gemm_grouped(bp(x), x.stride(0), bp(w), ip(seg), (int)w.size(0), rows, N, K, swiglu ? 1 : 0, bp(out), out.stride(0),
+                           cur_stream(), ipo(gather), x.size(0), ipo(scatter)), "gemm_grouped");
+  return out;
+}
+
+std::vector<at::Tensor> moe_route(const at::Tensor& ids, const at::Tensor& table, int64_t E) {
+  CHECK_CUDA(ids); CHECK_I32(ids); CHECK_CONTIG(ids); CHECK_CUDA(table); CHECK_I32(table); CHECK_CONTIG(table);
+  TORCH_CHECK(table.dim() == 2 && E >= 1, "table must be int32 [vocab, top]");
+  const long T = ids.numel();
+  const int top = table.size(1);
+  at::Tensor seg = at::empty({E + 1}, ids.options());
+  at::Tensor order = at::empty({T * top}, ids.options());
+  CHECK_RC(lk_moe_route(ip(ids), ip(table), (int)table.size(0), top, (int)E, (int)T, seg.data_ptr<int>(), order.data_ptr<int>(),
+                        cur_stream()), "moe_route");
+  return {seg, order};
+}
+
+at::Tensor moe_gemm(const at::Tensor& x, const at::Tensor& order, const at::Tensor& seg, const at::Tensor& w, int64_t top, bool act) {
+  CHECK_CUDA(x); CHECK_LASTDIM(x); CHECK_CUDA(w); CHECK_CONTIG(w); CHECK_CUDA(order); CHECK_I32(order); CHECK_CONTIG(order);
+  CHECK_CUDA(seg); CHECK_I32(seg); CHECK_CONTIG(seg);
+  const int esz = esz_of(x, "x");
+  same_type(w, x, "w");
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 3 && w.size(2) == x.size(1) && seg.numel() == w.size(0) + 1 && top >= 1, "x [rows, K], w [E, N, K]");
+  const long pairs = order.numel();
+  TORCH_CHECK(act ? x.size(0) * top == pairs : x.size(0) == pairs, "rows of x: tokens (act) or sorted pairs");
+  const int N = w.size(1);
+  at::Tensor out = at::empty({pairs, act ? N / 2 : N}, x.options());
+  CHECK_RC(lk_moe_gemm(x.data_ptr(), x.stride(0), ip(order), ip(seg), (int)w.size(0), (int)top, pairs, w.data_ptr(), N, (int)w.size(2),
+                       act ? 1 : 0, out.data_ptr(), out.stride(0), esz, cur_stream()), "moe_gemm");
+  return out;
 }
 
 }  // namespace
@@ -1533,6 +1681,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("normrope_kv_write", &normrope_kv_write);
   m.def("sinkattn_prefill", &sinkattn_prefill);
   m.def("sinkattn_decode", &sinkattn_decode);
+  m.def("stream_gated_norm", &stream_gated_norm);
+  m.def("rms_cols", &rms_cols);
+  m.def("rot_kv_write", &rot_kv_write);
+  m.def("pool_kv_write", &pool_kv_write);
+  m.def("moe_route", &moe_route);
+  m.def("gemm_grouped", &gemm_grouped);
+  m.def("gemm_grouped_supported", [](int64_t N, int64_t K, bool swiglu) { return lk_gemm_grouped_supported((int)N, (int)K, swiglu ? 1 : 0) != 0; });
+  m.def("moe_gemm", &moe_gemm);
   m.def("window_mark", [](int64_t id) { CHECK_RC(lk_window_mark((int)id, cur_stream()), "window_mark"); });
   m.def("debug_invalid_launch", []() { CHECK_RC(lk_debug_invalid_launch(cur_stream()), "debug_invalid_launch"); });
   // a HIP stream restricted to the CUs of a bit mask (32 CUs per word): two kernels that

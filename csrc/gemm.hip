@@ -120,7 +120,8 @@ constexpr int kSysCoherent = 1 | 16;  // buffer cache policy sc0 | sc1: past L1 
 
 // SC: this instantiation applies the folded-RMSNorm row scale (LkEpi::ss_in set): only those
 // carry the partial-sum prefetch registers through the K loop
-template <int NF, int EPI, int PH, int PRIO, bool SC>
+// GS (grouped form): X rows may be gathered and out rows scattered through LkEpi::gather / scatter
+template <int NF, int EPI, int PH, int PRIO, bool SC, bool GS = false>
 __device__ __forceinline__ void gemm8_body(const bf16_t* __restrict__ X, long ldx, const bf16_t* __restrict__ W,
                                            const bf16_t* __restrict__ bias, int M, int K, int I,
                                            bf16_t* __restrict__ out, long ldo, int TM, int TN, int group_m,
@@ -191,7 +192,7 @@ __device__ __forceinline__ void gemm8_body(const bf16_t* __restrict__ X, long ld
   // buffer_load ... lds through wave-uniform descriptors: fixed 32-bit per-lane row offsets, the
   // K offset in an SGPR, rows past M read as zeros by the descriptor's range check.
   const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
-      (void*)X, (short)0, (int)min((long)M * ldx * 2, 0x7FFFFFF0L), 0x00020000);
+      (void*)X, (short)0, (int)min((long)(GS && ea.gather ? ea.x_rows : M) * ldx * 2, 0x7FFFFFF0L), 0x00020000);
   const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
       (void*)W, (short)0, (int)min((long)(EPI == EPI_SWIGLU ? 2 * I : TN * BN) * K * 2, 0x7FFFFFF0L), 0x00020000);
   const int lr = lane >> 3, lc = lane & 7;
@@ -202,7 +203,13 @@ __device__ __forceinline__ void gemm8_body(const bf16_t* __restrict__ X, long ld
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int s = 16 * w + 8 * i + lr;
-      aoff[h][i] = (unsigned)(((long)tm * kBM + a_row(h, s)) * ldx * 2) + ((lc ^ swz(s)) << 4);
+      if constexpr (GS) {  // a gathered source row; tile rows past the expert's end point behind the descriptor's range
+        const int tr = tm * kBM + a_row(h, s);
+        const int src = tr < M ? (ea.gather ? ea.gather[tr] : tr) : -1;
+        aoff[h][i] = src >= 0 ? (unsigned)((long)src * ldx * 2) + ((lc ^ swz(s)) << 4) : 0xFFFFFF00u;
+      } else {
+        aoff[h][i] = (unsigned)(((long)tm * kBM + a_row(h, s)) * ldx * 2) + ((lc ^ swz(s)) << 4);
+      }
     }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
@@ -479,19 +486,25 @@ __device__ __forceinline__ void gemm8_body(const bf16_t* __restrict__ X, long ld
   // the 4 columns 32 + 4g .. +3.  (An LDS-staged whole-row store variant measured 0.98-1.04x
   // and raised every instantiation's VGPRs; removed: profiles/r4_kernels/README.md.)
   constexpr int OW = EPI == EPI_SWIGLU ? 128 : BN;  // output columns of the tile
+  auto out_row = [&](int lrow) -> long {
+    if constexpr (GS) {
+      if (ea.scatter) return (long)ea.scatter[tm * kBM + lrow];
+    }
+    return (long)(tm * kBM + lrow);
+  };
   auto emit8 = [&](int lrow, int lcol, const float (&y)[8]) {  // lcol: multiple of 8
     uint4_t pk;
     pk.x = pack_bf2(y[0], y[1]);
     pk.y = pack_bf2(y[2], y[3]);
     pk.z = pack_bf2(y[4], y[5]);
     pk.w = pack_bf2(y[6], y[7]);
-    *reinterpret_cast<uint4_t*>(out + (long)(tm * kBM + lrow) * ldo + (long)tn * OW + lcol) = pk;
+    *reinterpret_cast<uint4_t*>(out + out_row(lrow) * ldo + (long)tn * OW + lcol) = pk;
   };
   auto emit4 = [&](int lrow, int lcol, const float (&y)[4]) {  // lcol: multiple of 4
     uint2 pk;
     pk.x = pack_bf2(y[0], y[1]);
     pk.y = pack_bf2(y[2], y[3]);
-    *reinterpret_cast<uint2*>(out + (long)(tm * kBM + lrow) * ldo + (long)tn * OW + lcol) = pk;
+    *reinterpret_cast<uint2*>(out + out_row(lrow) * ldo + (long)tn * OW + lcol) = pk;
   };
   float scm[8];  // this lane's 8 row scales (1 unless the folded-norm scale applies)
 #pragma unroll
@@ -860,6 +873,54 @@ int group_rows() {
   return g;
 }
 
+// Grouped form for experts: the rows of X (and of out) are sorted by expert, rows seg[e] .. seg[e + 1] belong to expert e
+// whose weights are W + e * N * K.  Every expert is an ordinary GEMM of its own row count on the body above; a workgroup
+// finds its (expert, tile) by walking seg[] on the device, so the launch needs nothing from the host: the grid is the
+// upper bound (rows / 256 + E) * TN and surplus workgroups leave at once.  Rows past an expert's end read zeros through
+// the buffer descriptor's range check and are not stored.  gather (or null): X row of every sorted row (the experts'
+// inputs are then read in place instead of from a sorted copy); scatter (or null): out row of every sorted row.
+template <int NF, int EPI>
+__global__ __launch_bounds__(512, 1) void gemm_grouped_kernel(const bf16_t* __restrict__ X, long ldx,
+                                                              const bf16_t* __restrict__ W, const int* __restrict__ seg,
+                                                              int E, int N, int K, int I, bf16_t* __restrict__ out, long ldo,
+                                                              int TN, int group_m, const int* __restrict__ gather, long x_rows,
+                                                              const int* __restrict__ scatter) {
+  int e = -1, tile = 0, r0 = 0, rows = 0, acc = 0;
+  for (int i = 0; i < E; ++i) {
+    const int a = seg[i], m = seg[i + 1] - a, nt = ((m + kBM - 1) / kBM) * TN;
+    if (e < 0 && (int)blockIdx.x < acc + nt) {
+      e = i;
+      tile = blockIdx.x - acc;
+      r0 = a;
+      rows = m;
+    }
+    acc += nt;
+  }
+  if (e < 0) return;   // the whole workgroup: nothing of the body has run
+  const SkArgs sk{0, 0, nullptr, nullptr, nullptr, 0};
+  LkEpi ea{};
+  ea.gather = gather ? gather + r0 : nullptr;     // indexed by the expert's own tile rows
+  ea.scatter = scatter ? scatter + r0 : nullptr;
+  ea.x_rows = x_rows;
+  gemm8_body<NF, EPI, 4, 0, false, true>(gather ? X : X + (long)r0 * ldx, ldx, W + (long)e * N * K, nullptr, rows, K, I,
+                                         scatter ? out : out + (long)r0 * ldo, ldo, (rows + kBM - 1) / kBM, TN, group_m, tile, 0,
+                                         K / kBK, 0, SK_FULL, 0, sk, ea);
+  wait_vm<0>();
+}
+
+template <int NF, int EPI>
+int launch_grouped(const bf16_t* x, long ldx, const bf16_t* w, const int* seg, int E, long rows, int N, int K, int I, bf16_t* out,
+                   long ldo, int TN, hipStream_t st, const int* gather, long x_rows, const int* scatter) {
+  constexpr int lds = 2 * Geo<NF>::BUF;
+  LK_SET_MAX_LDS((gemm_grouped_kernel<NF, EPI>), lds);
+  const long grid = ((rows + kBM - 1) / kBM + E) * TN;
+  if (grid > 2147483647L) return -1;
+  gemm_grouped_kernel<NF, EPI><<<dim3((unsigned)grid), 512, lds, st>>>(x, ldx, w, seg, E, N, K, I, out, ldo, TN, group_rows(),
+                                                                       gather, x_rows, scatter);
+  LK_CHECK_LAUNCH();
+  return 0;
+}
+
 int cu_count() {
   static const int cus = [] {
     int dev = 0, n = 256;
@@ -1042,6 +1103,25 @@ int lk_gemm_streamk(int mode) {
     }
   }
   return errs;
+}
+
+int lk_gemm_grouped_supported(int N, int K, int swiglu) {
+  if (K < 2 * kBK || K % kBK || N < 1) return 0;
+  if (swiglu) return N % 2 == 0 && (N / 2) % 128 == 0;
+  return N % 256 == 0 || N % 192 == 0;
+}
+
+// out[r] = epi(X[r] . W_e^T) for the rows r in [seg[e], seg[e + 1]) of every expert e: X [rows, K] sorted by expert (row
+// stride ldx), W [E, N, K] contiguous, out [rows, N] (SwiGLU: W_e = [gate rows | up rows], out [rows, N / 2]).
+int lk_gemm_grouped(const bf16_t* x, long ldx, const bf16_t* w, const int* seg, int E, long rows, int N, int K, int swiglu,
+                    bf16_t* out, long ldo, hipStream_t st, const int* gather, long x_rows, const int* scatter) {
+  if (rows <= 0) return 0;
+  if (E < 1 || (gather && x_rows < 1) || !lk_gemm_grouped_supported(N, K, swiglu) || ldx % 8 || ldo % 8 || reinterpret_cast<uintptr_t>(out) % 16 ||
+      reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(w) % 16)
+    return -1;
+  if (swiglu) return launch_grouped<4, EPI_SWIGLU>(x, ldx, w, seg, E, rows, N, K, N / 2, out, ldo, N / 256, st, gather, x_rows, scatter);
+  if (N % 256 == 0) return launch_grouped<4, EPI_NONE>(x, ldx, w, seg, E, rows, N, K, 0, out, ldo, N / 256, st, gather, x_rows, scatter);
+  return launch_grouped<3, EPI_NONE>(x, ldx, w, seg, E, rows, N, K, 0, out, ldo, N / 192, st, gather, x_rows, scatter);
 }
 
 int lk_gemm_supported(int M, int N, int K, int epi, int bn, int ks) {

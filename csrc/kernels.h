@@ -119,11 +119,22 @@ struct LkEpi {
   bf16_t* kc = nullptr;          // QKV: paged caches [num_blocks, hkv, bs, hd]
   bf16_t* vc = nullptr;
   int bs = 0, hq = 0, hkv = 0, hd = 0;
+  // grouped form only (gemm_grouped_kernel): tile row j of the expert reads X row gather[j] (null: row j of the
+  // expert's own rows) and writes out row scatter[j] (null: row j); x_rows = rows of X behind the gather
+  const int* gather = nullptr;
+  const int* scatter = nullptr;
+  long x_rows = 0;
 };
 // variant: K-loop schedule of gemm.hip (0 / 1 / 2), or 3 = gemm1w.hip (bn 256)
 int lk_gemm(const bf16_t* x, long ldx, const bf16_t* w, const bf16_t* bias, int M, int N, int K, int epi, int bn,
             int variant, bf16_t* out, long ldo, hipStream_t st, int ks = 1, float* ws = nullptr,
             const LkEpi* ea = nullptr);
+
+// grouped form of lk_gemm for rows sorted by expert (segment offsets on the device; weights [E, N, K]); no bias, epilogue
+// none or SwiGLU.  Needs K % 64 == 0, K >= 128, N % 256 or N % 192 == 0 (SwiGLU: N/2 % 128 == 0)
+int lk_gemm_grouped_supported(int N, int K, int swiglu);
+int lk_gemm_grouped(const bf16_t* x, long ldx, const bf16_t* w, const int* seg, int E, long rows, int N, int K, int swiglu,
+                    bf16_t* out, long ldo, hipStream_t st, const int* gather = nullptr, long x_rows = 0, const int* scatter = nullptr);
 
 // gemm1w.hip: the one-wave-per-SIMD bm x 256 prefill GEMM (hipBLASLt's gfx950 K-loop schedule,
 // every lk_gemm epilogue); lk_gemm routes variants 3 / 4 / 5 here (row tile bm = 256 / 192 / 128).
@@ -243,7 +254,7 @@ int lk_sigattn_decode(const void* q, long qs, const void* kc, const void* vc, co
 
 // csrc/ssm.hip: selective state-space mixer (sequences = rows [cu[s], cu[s+1]), state slot slots[s])
 int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const float* bias, void* state, const int* cu,
-                 const int* slots, const int* positions, int S, int max_len, void* out, long os, int esz,
+                 const int* slots, const int* positions, int S, int max_len, void* out, long os, int act, int esz,
                  hipStream_t st);
 int lk_ssm_scan(const void* xbc, long xs, const void* dt, long dts, int S, int heads, int P, int N, int groups,
                 const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu, const int* slots,
@@ -253,7 +264,7 @@ int lk_gated_group_rmsnorm(const float* y, long ys, const void* z, long zs, cons
 
 // csrc/stream_ln.hip: post-norm f32 stream (x <- LN(alpha x + ls * y) * w + b with an activation-dtype copy), token gather,
 // gated tanh-GELU of a fused [gate | up] projection, mean of two RMS-normed branches
-int lk_embed_stream(const int* ids, const void* tok, long V, long T, int W, float* x, void* copy, int esz, hipStream_t st);
+int lk_embed_stream(const int* ids, const void* tok, long V, long T, int W, float* x, void* copy, float scale, int esz, hipStream_t st);
 int lk_stream_layernorm(float* x, const void* y, long ys, int y_esz, const float* ls, float alpha, const float* w, const float* b,
                         float eps, const long* idx, long rows, void* out, long os, int out_esz, int W, hipStream_t st);
 int lk_gelu_tanh_mul(const void* gu, long gs, void* out, long os, long rows, int F, int esz, hipStream_t st);
@@ -276,14 +287,33 @@ int lk_head_norm_gate(const float* o, long os, const void* g, long gs, int g_esz
 int lk_tanh_(void* x, long xs, long T, int n, int esz, hipStream_t st);
 
 // csrc/attn_sink.hip: softmax attention with a sink and a position mask (0 causal, 1 chunks, 2 window) over the paged caches
-// K [NB, G, BS, dim], V [NB, G, vdim, BS]; q / k RMS norm + partial rotation, v norm and the cache write
+// K [NB, G, BS, dim], V [NB, G, vdim, BS], optionally beside pooled keys / values of whole blocks before a window (pkc, pvc,
+// pool); q / k RMS norm + partial rotation, v norm and the cache write
 int lk_normrope_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int vdim, int norm_dim, int norm_vdim, const float* qw,
                          const float* kw, int rot, const float* inv_freq, const int* positions, float eps, void* kc, void* vc,
                          const int* slots, int BS, int v_unit, int esz, hipStream_t st);
 int lk_sinkattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* cu_q,
                         const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H, int G, int dim, int vdim,
                         int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol, void* out,
-                        long os, int esz, hipStream_t st);
+                        long os, const void* pkc, const void* pvc, int pool, int esz, hipStream_t st);
 int lk_sinkattn_decode(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* ctx_lens,
                        int B, int Z, int H, int G, int dim, int vdim, int BS, const float* hscale, int mkind, int msize, int sink,
-                       const void* gate, long gs, int gcol, void* out, long os, float* part, int esz, hipStream_t st);
+                       const void* gate, long gs, int gcol, void* out, long os, float* part, const void* pkc, const void* pvc,
+                       int pool, int esz, hipStream_t st);
+
+// csrc/window_ops.hip: gated + normed sublayer result into the f32 stream (+ the next norm), RMS norm of a column block,
+// pair rotation + key assembly + paged K / V write, pooled (mean) keys / values of finished blocks
+int lk_stream_gated_norm(float* x, const void* y, long ys, int parts, const void* g, long gs, const float* gb, const float* wpost,
+                         const float* wnext, float eps, void* out, long os, long rows, int W, int esz, hipStream_t st);
+int lk_rms_cols(const void* u, long us, int n, const float* w, float eps, void* out, long os, long rows, int esz, hipStream_t st);
+int lk_rot_kv_write(void* q, long qs, int H, int qdim, const void* k, long ks, int G, int kdim, const void* sh, long shs, int sdim,
+                    const void* v, long vs, int vdim, int rot_off, int rot, const float* freq, float mag, const int* positions,
+                    void* kc, void* vc, const int* slots, int BS, int KD, int VD, long T, int esz, hipStream_t st);
+int lk_pool_kv_write(const void* kc, const void* vc, void* pkc, void* pvc, int P, const int* bt, int bt_stride, const int* ctx_lens,
+                     const int* cu_q, const int* slots, int row0, int S, int max_len, int G, int BS, int dim, int vdim, int esz,
+                     hipStream_t st);
+
+// csrc/moe.hip: experts chosen by a table of token ids: pairs sorted by expert on the device, grouped MFMA products
+int lk_moe_route(const int* ids, const int* table, int vocab, int top, int E, int T, int* seg, int* order, hipStream_t st);
+int lk_moe_gemm(const void* x, long xs, const int* order, const int* seg, int E, int top, long pairs, const void* w, int N, int K,
+                int act, void* out, long os, int esz, hipStream_t st);

@@ -2,7 +2,7 @@
 // along the recurrence:
 //
 //   u_t  = [z | x B C | dt]                       the input projection's row (bf16 or f32)
-//   xBC  = silu(causal_conv(x B C) + b)           per channel, `taps` wide, the last column is the
+//   xBC  = silu(causal_conv(x B C) + b)           per channel, `taps` wide (act = 0: without the SiLU), the last column is the
 //                                                 current token's; the taps - 1 inputs before a chunk
 //                                                 come from the sequence's conv state
 //   dt   = softplus(dt + dt_bias)                 f32, no clamp
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const T* __restrict__ u,
                                                         const T* __restrict__ state, const int* __restrict__ cu,
                                                         const int* __restrict__ slots,
                                                         const int* __restrict__ positions, T* __restrict__ out,
-                                                        long os) {
+                                                        long os, int act) {
   const int s = blockIdx.x, c = blockIdx.z * 256 + threadIdx.x;
   const int row0 = cu[s], len = cu[s + 1] - row0, slot = slots[s];
   const int i0 = blockIdx.y * kConvRows;
@@ -74,11 +74,11 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const T* __restrict__ u,
         acc += wk[k] * v;
       }
     }
-    stf<T>(out + (long)(row0 + i) * os + c, silu_f<sizeof(T) == 4>(acc));
+    stf<T>(out + (long)(row0 + i) * os + c, act ? silu_f<sizeof(T) == 4>(acc) : acc);
   }
 }
 
-// The same for taps <= 4 with 16-byte accesses: a thread owns EV adjacent channels and walks its 16
+// The same for taps <= 4 with 16-byte accesses: a thread owns EV adjacent channels and walks its `rows`
 // tokens with the three previous inputs in registers (weights right-aligned in a 4-tap window, the
 // unused leading taps zero), so every input row is read once per tile instead of once per tap.
 // Needs C % EV == 0 and 16-byte aligned rows of u, out and the state.
@@ -88,13 +88,13 @@ __global__ __launch_bounds__(256) void conv_silu_vec_kernel(const T* __restrict_
                                                             const T* __restrict__ state, const int* __restrict__ cu,
                                                             const int* __restrict__ slots,
                                                             const int* __restrict__ positions, T* __restrict__ out,
-                                                            long os) {
+                                                            long os, int act, int rows) {
   constexpr int EV = 16 / sizeof(T);
   const int s = blockIdx.x, c0 = (blockIdx.z * 256 + threadIdx.x) * EV;
   const int row0 = cu[s], len = cu[s + 1] - row0, slot = slots[s];
-  const int i0 = blockIdx.y * kConvRows;
+  const int i0 = blockIdx.y * rows;
   if (c0 >= C || i0 >= len) return;
-  const int i1 = min(len, i0 + kConvRows);
+  const int i1 = min(len, i0 + rows);
   auto ldrow = [&](const T* p, float (&f)[EV]) {
     if constexpr (sizeof(T) == 2) {
       load8(p, f);
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void conv_silu_vec_kernel(const T* __restrict_
 #pragma unroll
     for (int e = 0; e < EV; ++e) {
       const float acc = b[e] + wk[0][e] * win[0][e] + wk[1][e] * win[1][e] + wk[2][e] * win[2][e] + wk[3][e] * cur[e];
-      r[e] = silu_f<sizeof(T) == 4>(acc);
+      r[e] = act ? silu_f<sizeof(T) == 4>(acc) : acc;
       win[0][e] = win[1][e];
       win[1][e] = win[2][e];
       win[2][e] = cur[e];
@@ -582,7 +582,7 @@ int scan_t(const T* xbc, long xs, const T* dtp, long dts, int S, int heads, int 
 }  // namespace
 
 int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const float* bias, void* state, const int* cu,
-                 const int* slots, const int* positions, int S, int max_len, void* out, long os, int esz,
+                 const int* slots, const int* positions, int S, int max_len, void* out, long os, int act, int esz,
                  hipStream_t st) {
   if (S <= 0 || max_len <= 0) return 0;
   if (taps < 1 || taps > kMaxTaps || C <= 0) return -1;
@@ -590,13 +590,17 @@ int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const 
   const int ev = 16 / esz;
   const auto a16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
   if (taps <= 4 && C % ev == 0 && us % ev == 0 && os % ev == 0 && a16(u) && a16(out) && a16(state)) {
-    dim3 gv(S, (max_len + kConvRows - 1) / kConvRows, (C / ev + 255) / 256);
+    const int cblocks = (C / ev + 255) / 256;
+    // tokens per workgroup (a kernel argument: tiles of 4 tokens were tried for steps of few, long sequences, where 16-token
+    // tiles leave a chip of 256 CUs a handful of waves each, and measured slower: 79 us against 61 us at 4 x 1,024 x 2,048)
+    const int rows = kConvRows;
+    dim3 gv(S, (max_len + rows - 1) / rows, cblocks);
     if (esz == 2)
       conv_silu_vec_kernel<bf16_t><<<gv, 256, 0, st>>>((const bf16_t*)u, us, C, taps, w, bias, (const bf16_t*)state, cu,
-                                                       slots, positions, (bf16_t*)out, os);
+                                                       slots, positions, (bf16_t*)out, os, act, rows);
     else
       conv_silu_vec_kernel<float><<<gv, 256, 0, st>>>((const float*)u, us, C, taps, w, bias, (const float*)state, cu, slots,
-                                                      positions, (float*)out, os);
+                                                      positions, (float*)out, os, act, rows);
     LK_CHECK_LAUNCH();
     if (taps > 1) {
       if (esz == 2) conv_state_kernel<bf16_t><<<g2, 256, 0, st>>>((const bf16_t*)u, us, C, taps, (bf16_t*)state, cu, slots, positions);
@@ -607,12 +611,12 @@ int lk_conv_silu(const void* u, long us, int C, int taps, const float* w, const 
   }
   if (esz == 2) {
     conv_silu_kernel<bf16_t><<<grid, 256, 0, st>>>((const bf16_t*)u, us, C, taps, w, bias, (const bf16_t*)state, cu,
-                                                   slots, positions, (bf16_t*)out, os);
+                                                   slots, positions, (bf16_t*)out, os, act);
     LK_CHECK_LAUNCH();
     if (taps > 1) conv_state_kernel<bf16_t><<<g2, 256, 0, st>>>((const bf16_t*)u, us, C, taps, (bf16_t*)state, cu, slots, positions);
   } else {
     conv_silu_kernel<float><<<grid, 256, 0, st>>>((const float*)u, us, C, taps, w, bias, (const float*)state, cu, slots,
-                                                  positions, (float*)out, os);
+                                                  positions, (float*)out, os, act);
     LK_CHECK_LAUNCH();
     if (taps > 1) conv_state_kernel<float><<<g2, 256, 0, st>>>((const float*)u, us, C, taps, (float*)state, cu, slots, positions);
   }

@@ -27,18 +27,18 @@ LK_DEVICE void stv<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
 template <>
 LK_DEVICE void stv<float>(float* p, float v) { *p = v; }
 
-// one workgroup per token: x f32 [T, W] and (copy != null) the same values in the table's dtype
+// one workgroup per token: x f32 [T, W] = row * scale and (copy != null) the same values in the table's dtype
 template <typename T>
 __global__ __launch_bounds__(256) void embed_stream_kernel(const int* __restrict__ ids, const T* __restrict__ tok, long V, int W,
-                                                           float* __restrict__ x, T* __restrict__ copy) {
+                                                           float* __restrict__ x, T* __restrict__ copy, float scale) {
   const long t = blockIdx.x;
   long id = ids[t];
   id = id < 0 ? 0 : (id >= V ? V - 1 : id);
   const T* src = tok + id * W;
   for (int c = threadIdx.x; c < W; c += 256) {
-    const T v = src[c];
-    x[t * W + c] = ldv<T>(&v);
-    if (copy) copy[t * W + c] = v;
+    const float v = ldv<T>(src + c) * scale;
+    x[t * W + c] = v;
+    if (copy) stv<T>(copy + t * W + c, v);
   }
 }
 
@@ -190,10 +190,11 @@ int launch_ln(float* x, const void* y, long ys, const float* ls, float alpha, co
 
 }  // namespace
 
-int lk_embed_stream(const int* ids, const void* tok, long V, long T, int W, float* x, void* copy, int esz, hipStream_t st) {
+int lk_embed_stream(const int* ids, const void* tok, long V, long T, int W, float* x, void* copy, float scale, int esz,
+                    hipStream_t st) {
   if (T <= 0) return 0;
-  if (esz == 2) embed_stream_kernel<bf16_t><<<(unsigned)T, 256, 0, st>>>(ids, (const bf16_t*)tok, V, W, x, (bf16_t*)copy);
-  else embed_stream_kernel<float><<<(unsigned)T, 256, 0, st>>>(ids, (const float*)tok, V, W, x, (float*)copy);
+  if (esz == 2) embed_stream_kernel<bf16_t><<<(unsigned)T, 256, 0, st>>>(ids, (const bf16_t*)tok, V, W, x, (bf16_t*)copy, scale);
+  else embed_stream_kernel<float><<<(unsigned)T, 256, 0, st>>>(ids, (const float*)tok, V, W, x, (float*)copy, scale);
   LK_CHECK_LAUNCH();
   return 0;
 }
