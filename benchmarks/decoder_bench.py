@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of the hybrid decoders (Lebepel; Pemidra with ``--models pemidra,lebepel``)
-beside a Llama decoder of the same width, depth, heads, head size, feed-forward and vocabulary (random
+"""Prefill and decode throughput of the hybrid decoders (Lebepel; Pemidra with ``--models pemidra,lebepel``;
+Fusasun with ``--models fusasun,llama``) beside a Llama decoder of the same width, depth, heads, head size, feed-forward and vocabulary (random
 weights, bf16, one GPU), all through the same engine: prefill = S fresh prompts of L tokens in one step, decode = B sequences at
 context C, one token each per step (hipGraph replay).  ``bench.py --decoder-bench`` runs this.
 
@@ -32,8 +32,8 @@ VOCAB = 32768
 
 def models(width: int, which: str, device):
     from llm_kubernetes_minikube_sharp4dev_amd.models import build_decoder
-    from llm_kubernetes_minikube_sharp4dev_amd.models.configs import (LebepelConfig, PemidraConfig, decoder_config, lebepel_layers,
-                                                                      pemidra_layers)
+    from llm_kubernetes_minikube_sharp4dev_amd.models.configs import (FusasunConfig, LebepelConfig, PemidraConfig, decoder_config,
+                                                                      fusasun_layers, lebepel_layers, pemidra_layers)
 
     L, H, G, D, FF, sh, sp, sn, sg = SIZES[width]
     if which == "lebepel":
@@ -44,6 +44,13 @@ def models(width: int, which: str, device):
         # feed-forward) in turn; the same heads and head size for every mixer, two-layer projections of rank 128
         cfg = PemidraConfig(f"pemidra-w{width}", VOCAB, width, pemidra_layers(L, H, D, FF, kv_heads=G, chunk=256, lora=128),
                             postln_alpha=2.0)
+    elif which == "fusasun":
+        # pooled-window attention (window 512, blocks of 64) and latent attention (window 512, latent 512 + 64 rotated)
+        # in turn, the same heads and head size; 16 experts of half the dense feed-forward, two per token: the
+        # products a token runs are those of the dense model
+        cfg = FusasunConfig(f"fusasun-w{width}", VOCAB, width,
+                            fusasun_layers(L, H, D, FF // 2, 16, 2, kv_heads=G, window=512, pool=64, rot_dim=64,
+                                           q_rank=max(512, width // 2), kv_rank=512), embed_scale=1.0, canon_taps=4)
     else:
         cfg = decoder_config("llama-3-8b", num_layers=L, hidden=width, num_heads=H, num_kv_heads=G, head_dim=D,
                              intermediate=FF, vocab_size=VOCAB, max_position=8192)
@@ -100,7 +107,7 @@ def run(width: int, which: str, a) -> dict:
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--sizes", default="1024,2048,4096")
-    ap.add_argument("--models", default="lebepel,llama", help="comma list of lebepel, pemidra, llama")
+    ap.add_argument("--models", default="lebepel,llama", help="comma list of lebepel, pemidra, fusasun, llama")
     ap.add_argument("--prefill-seqs", type=int, default=4)
     ap.add_argument("--prefill-len", type=int, default=1024)
     ap.add_argument("--decode-batch", type=int, default=64)
