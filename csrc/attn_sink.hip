@@ -15,6 +15,11 @@
 // second cache pair of the same layout, entry b at the logical position b of the sequence's block table, so
 // the pass over them is the pass over the window with other pointers and the bound "b < blocks seen".
 //
+// Kept first positions (window masks without pooling, keep > 0): positions below `keep` stay visible to every
+// later query, at their true places; the ones the window has left are one more pass over the first cache pages.
+// cap > 0: a score s enters the softmax as cap * tanh(s / cap).  The optional gate is one sigmoid per head or
+// (gelem) one per output element.
+//
 // lk_normrope_kv_write prepares the operands in f32: q and k RMS-normed per head with a weight shared by
 // the heads, their first `rot` dimensions rotated by the position (dimension i pairs with i + rot / 2),
 // v divided by its RMS; q in place, k and v into the cache.
@@ -53,6 +58,9 @@ struct SinkParams {
   const void* pkc;      // pooled K / V caches (pool > 0)
   const void* pvc;
   int pool;
+  int keep;             // window masks: positions below `keep` stay visible behind the window
+  float cap;            // > 0: scores become cap * tanh(score / cap)
+  int gelem;            // the gate has one column per output element (gcol + h * vdim + d) instead of one per head
 };
 
 LK_DEVICE int blocks_seen(int qpos, int msize, int pool) { return max(0, qpos - msize + 1) / pool; }
@@ -74,6 +82,13 @@ template <bool EXACT>
 LK_DEVICE float exp_f(float x) {
   if constexpr (EXACT) return expf(x);
   else return __expf(x);
+}
+
+// cap * tanh(s / cap); icap = 1 / cap
+template <bool EXACT>
+LK_DEVICE float cap_f(float s, float cap, float icap) {
+  if constexpr (EXACT) return cap * tanhf(s * icap);
+  else return cap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * s * icap)));
 }
 
 // The columns of this wave against the 32-key steps step0, step0 + stride, ... of keys [k0, k1): k0 is a
@@ -133,6 +148,7 @@ LK_DEVICE void sink_run(const SinkParams& p, const uint4_t (&qf)[PAD / (4 * El<T
     float sc[2][4];
     bool ok[2][4];
     float mx = kNegBig;
+    const float icap = p.cap > 0.f ? 1.f / p.cap : 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -140,6 +156,7 @@ LK_DEVICE void sink_run(const SinkParams& p, const uint4_t (&qf)[PAD / (4 * El<T
         const int key = kb + 8 * g + 4 * t + j;
         ok[t][j] = cvalid && key <= qpos && key >= klo && key < k1;
         sc[t][j] = c[t][j] * hs;
+        if (p.cap > 0.f) sc[t][j] = cap_f<!BF>(sc[t][j], p.cap, icap);
         if (ok[t][j]) mx = fmaxf(mx, sc[t][j]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -232,12 +249,24 @@ LK_DEVICE void merge_waves(float& m, float& l, floatx4 (&o)[VT], float (&red)[3]
   }
 }
 
+// the head's gate (1 when there is none, or when the gate is per element)
 template <typename T>
 LK_DEVICE float gate_of(const SinkParams& p, long row, int head) {
-  if (!p.gate) return 1.f;
+  if (!p.gate || p.gelem) return 1.f;
   const float gv = El<T>::ld(reinterpret_cast<const T*>(p.gate) + row * p.gs + p.gcol + head);
   return 1.f / (1.f + expf(-gv));
 }
+
+// the gate of output element vd of a head (1 unless the gate is per element)
+template <typename T>
+LK_DEVICE float gate_el(const SinkParams& p, long row, int head, int vd) {
+  if (!p.gate || !p.gelem) return 1.f;
+  const float gv = El<T>::ld(reinterpret_cast<const T*>(p.gate) + row * p.gs + p.gcol + (long)head * p.vdim + vd);
+  return 1.f / (1.f + expf(-gv));
+}
+
+// the positions below `keep` that lie behind the window of a query whose first visible key is klo
+LK_DEVICE int kept_keys(const SinkParams& p, int klo) { return p.keep > 0 ? min(p.keep, klo) : 0; }
 
 // ---- prefill: blockIdx.x = head, blockIdx.y walks the tile list (16 queries of one sequence each).
 // WT = false: a workgroup owns one tile, its 4 waves take every fourth 32-key step and are merged (long key
@@ -280,6 +309,13 @@ __global__ __launch_bounds__(256) void sinkattn_prefill_kernel(SinkParams p, con
       sink_run<T, PAD>(pooled_view(p), qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, nbt, WT ? 0 : w, WT ? 1 : 4,
                        cvalid, blocks_seen(qpos, p.msize, p.pool) - 1, 0, p.hscale[head], m, l, o);
   }
+  {
+    // kept first positions behind the window: the tile's last query has the latest window, so it bounds the pass
+    const int nk = kept_keys(p, first_key(k1 - 1, p.mkind, p.msize));
+    if (nk > 0)
+      sink_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, nk, WT ? 0 : w, WT ? 1 : 4, cvalid,
+                       kept_keys(p, first_key(qpos, p.mkind, p.msize)) - 1, 0, p.hscale[head], m, l, o);
+  }
   if constexpr (WT) {
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -295,7 +331,7 @@ __global__ __launch_bounds__(256) void sinkattn_prefill_kernel(SinkParams p, con
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int vd = vt * 16 + 4 * g + j;
-        if (vd < p.vdim) El<T>::st(orow + vd, o[vt][j] * f);
+        if (vd < p.vdim) El<T>::st(orow + vd, o[vt][j] * f * gate_el<T>(p, qbeg + qi, head, vd));
       }
   }
 }
@@ -325,15 +361,20 @@ __global__ __launch_bounds__(256) void sinkattn_decode_kernel(SinkParams p, cons
   float m = p.sink ? 0.f : kNegBig, l = 0.f;
   const int klo = first_key(ctx - 1, p.mkind, p.msize), k0 = klo & ~31;
   // the key splits share the window's 32-key steps and, behind them, the steps over the pooled blocks
+  // and, behind those, the steps over the kept first positions that the window has left
   const int nb = p.pool > 0 ? blocks_seen(ctx - 1, p.msize, p.pool) : 0;
-  const int nwin = (ctx - k0 + 31) / 32, nsteps = nwin + (nb + 31) / 32, spz = (nsteps + Z - 1) / Z;
+  const int nk = kept_keys(p, klo);
+  const int nwin = (ctx - k0 + 31) / 32, e1 = nwin + (nb + 31) / 32, nsteps = e1 + (nk + 31) / 32, spz = (nsteps + Z - 1) / Z;
   const int s0 = z * spz, s1 = min(nsteps, s0 + spz);
   if (s0 < min(s1, nwin))
     sink_run<T, PAD>(p, qf, kvh, p.bt + (long)b * p.bt_stride, k0 + 32 * s0, min(ctx, k0 + 32 * min(s1, nwin)), w, 4, cvalid, ctx - 1,
                      klo, p.hscale[head], m, l, o);
-  if (max(s0, nwin) < s1)
-    sink_run<T, PAD>(pooled_view(p), qf, kvh, p.bt + (long)b * p.bt_stride, 32 * (max(s0, nwin) - nwin), min(nb, 32 * (s1 - nwin)), w, 4,
-                     cvalid, nb - 1, 0, p.hscale[head], m, l, o);
+  if (max(s0, nwin) < min(s1, e1))
+    sink_run<T, PAD>(pooled_view(p), qf, kvh, p.bt + (long)b * p.bt_stride, 32 * (max(s0, nwin) - nwin), min(nb, 32 * (min(s1, e1) - nwin)),
+                     w, 4, cvalid, nb - 1, 0, p.hscale[head], m, l, o);
+  if (max(s0, e1) < s1)
+    sink_run<T, PAD>(p, qf, kvh, p.bt + (long)b * p.bt_stride, 32 * (max(s0, e1) - e1), min(nk, 32 * (s1 - e1)), w, 4, cvalid, nk - 1, 0,
+                     p.hscale[head], m, l, o);
   merge_waves<EXACT, VT>(m, l, o, red, ml);
   if (w == 0 && cvalid) {
     if (Z == 1) {
@@ -344,7 +385,7 @@ __global__ __launch_bounds__(256) void sinkattn_decode_kernel(SinkParams p, cons
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int vd = vt * 16 + 4 * g + j;
-          if (vd < p.vdim) El<T>::st(out + (long)b * os + (long)head * p.vdim + vd, o[vt][j] * f);
+          if (vd < p.vdim) El<T>::st(out + (long)b * os + (long)head * p.vdim + vd, o[vt][j] * f * gate_el<T>(p, b, head, vd));
         }
     } else {
       float* pp = part + (((long)b * p.H + head) * Z + z) * (p.vdim + 2);
@@ -377,7 +418,7 @@ __global__ __launch_bounds__(256) void sinkattn_reduce_kernel(SinkParams p, cons
   for (int vd = threadIdx.x; vd < p.vdim; vd += 256) {
     float s = 0.f;
     for (int z = 0; z < Z; ++z) s += pp[(long)z * (p.vdim + 2) + vd] * exp_f<EXACT>(pp[(long)z * (p.vdim + 2) + p.vdim] - M);
-    El<T>::st(out + (long)b * os + (long)head * p.vdim + vd, s * f);
+    El<T>::st(out + (long)b * os + (long)head * p.vdim + vd, s * f * gate_el<T>(p, b, head, vd));
   }
 }
 
@@ -470,7 +511,8 @@ bool shape_ok(const SinkParams& p, int esz) {
   const int ev = 16 / esz;
   return p.H > 0 && p.G > 0 && p.H % p.G == 0 && p.dim > 0 && p.vdim > 0 && p.dim % ev == 0 && p.vdim % ev == 0 && p.BS % 16 == 0 &&
          pad_of(p.dim, p.vdim) != 0 && p.mkind >= 0 && p.mkind <= 2 && (p.mkind == 0 || p.msize >= 1) && p.pool >= 0 &&
-         (p.pool == 0 || (p.mkind == 2 && p.pkc != nullptr && p.pvc != nullptr));
+         (p.pool == 0 || (p.mkind == 2 && p.pkc != nullptr && p.pvc != nullptr)) && p.keep >= 0 &&
+         (p.keep == 0 || (p.mkind == 2 && p.pool == 0)) && p.cap >= 0.f;
 }
 
 template <typename T, int PAD>
@@ -521,11 +563,11 @@ int decode_t(const SinkParams& p, const int* ctx, int B, int Z, void* out, long 
 
 SinkParams make_params(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, int H, int G, int dim,
                        int vdim, int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol,
-                       const void* pkc, const void* pvc, int pool) {
+                       const void* pkc, const void* pvc, int pool, int keep, float cap, int gelem) {
   SinkParams p;
   p.q = q; p.qs = qs; p.kc = kc; p.vc = vc; p.bt = bt; p.bt_stride = bt_stride;
   p.H = H; p.G = G; p.dim = dim; p.vdim = vdim; p.BS = BS; p.hscale = hscale; p.mkind = mkind; p.msize = msize; p.sink = sink;
-  p.gate = gate; p.gs = gs; p.gcol = gcol; p.pkc = pkc; p.pvc = pvc; p.pool = pool;
+  p.gate = gate; p.gs = gs; p.gcol = gcol; p.pkc = pkc; p.pvc = pvc; p.pool = pool; p.keep = keep; p.cap = cap; p.gelem = gelem;
   return p;
 }
 
@@ -551,9 +593,10 @@ int lk_normrope_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int 
 int lk_sinkattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* cu_q,
                         const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H, int G, int dim, int vdim,
                         int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol, void* out,
-                        long os, const void* pkc, const void* pvc, int pool, int esz, hipStream_t st) {
+                        long os, const void* pkc, const void* pvc, int pool, int keep, float cap, int gelem, int esz, hipStream_t st) {
   if (ntiles <= 0) return 0;
-  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol, pkc, pvc, pool);
+  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol, pkc, pvc,
+                                   pool, keep, cap, gelem);
   if (!shape_ok(p, esz)) return -1;
   return esz == 2 ? prefill_t<bf16_t>(p, cu_q, ctx_lens, tile_seq, tile_q0, ntiles, out, os, st)
                   : prefill_t<float>(p, cu_q, ctx_lens, tile_seq, tile_q0, ntiles, out, os, st);
@@ -562,9 +605,10 @@ int lk_sinkattn_prefill(const void* q, long qs, const void* kc, const void* vc, 
 int lk_sinkattn_decode(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* ctx_lens,
                        int B, int Z, int H, int G, int dim, int vdim, int BS, const float* hscale, int mkind, int msize, int sink,
                        const void* gate, long gs, int gcol, void* out, long os, float* part, const void* pkc, const void* pvc,
-                       int pool, int esz, hipStream_t st) {
+                       int pool, int keep, float cap, int gelem, int esz, hipStream_t st) {
   if (B <= 0) return 0;
-  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol, pkc, pvc, pool);
+  const SinkParams p = make_params(q, qs, kc, vc, bt, bt_stride, H, G, dim, vdim, BS, hscale, mkind, msize, sink, gate, gs, gcol, pkc, pvc,
+                                   pool, keep, cap, gelem);
   if (!shape_ok(p, esz) || Z < 1 || (Z > 1 && part == nullptr)) return -1;
   return esz == 2 ? decode_t<bf16_t>(p, ctx_lens, B, Z, out, os, part, st) : decode_t<float>(p, ctx_lens, B, Z, out, os, part, st);
 }

@@ -1445,7 +1445,7 @@ void normrope_kv_write(at::Tensor& qkv, int64_t H, int64_t G, int64_t dim, int64
 }
 
 const void* gate_rows(const c10::optional<at::Tensor>& gate, const at::Tensor& q, int64_t gate_col, int64_t H, long* gs) {
-  if (!gate) return nullptr;
+  if (!gate) return nullptr;   // H: the gate's columns (one per head, or one per output element)
   check_rows(*gate, q.size(0), gate_col + H, "gate");
   same_type(*gate, q, "gate");
   TORCH_CHECK(gate_col >= 0, "gate_col");
@@ -1469,7 +1469,8 @@ void sinkattn_prefill(const at::Tensor& q, const at::Tensor& kc, const at::Tenso
                       const at::Tensor& ctx, const at::Tensor& tile_seq, const at::Tensor& tile_q0, int64_t H, int64_t G, int64_t dim,
                       int64_t vdim, const at::Tensor& hscale, int64_t mkind, int64_t msize, bool sink,
                       const c10::optional<at::Tensor>& gate, int64_t gate_col, at::Tensor& out,
-                      const c10::optional<at::Tensor>& pkc, const c10::optional<at::Tensor>& pvc, int64_t pool) {
+                      const c10::optional<at::Tensor>& pkc, const c10::optional<at::Tensor>& pvc, int64_t pool, int64_t keep_first,
+                      double softcap, bool gate_elem) {
   CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(out); CHECK_LASTDIM(out);
   const int esz = esz_of(q, "q");
   const void *pkp = nullptr, *pvp = nullptr;
@@ -1483,18 +1484,20 @@ void sinkattn_prefill(const at::Tensor& q, const at::Tensor& kc, const at::Tenso
   TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1 && bt.size(0) >= cu_q.numel() - 1 && ctx.numel() >= cu_q.numel() - 1 &&
               tile_q0.numel() == tile_seq.numel(), "block tables / lengths / tiles");
   long gs = 0;
-  const void* gp = gate_rows(gate, q, gate_col, H, &gs);
+  const void* gp = gate_rows(gate, q, gate_col, gate_elem ? H * vdim : H, &gs);
+  TORCH_CHECK(keep_first >= 0 && softcap >= 0, "keep_first / softcap");
   CHECK_RC(lk_sinkattn_prefill(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), (int)bt.stride(0), ip(cu_q), ip(ctx),
                                ip(tile_seq), ip(tile_q0), (int)tile_seq.numel(), (int)H, (int)G, (int)dim, (int)vdim, (int)kc.size(2),
                                fp(hscale, H, "hscale"), (int)mkind, (int)msize, sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(),
-                               out.stride(0), pkp, pvp, (int)pool, esz, cur_stream()), "sinkattn_prefill");
+                               out.stride(0), pkp, pvp, (int)pool, (int)keep_first, (float)softcap, gate_elem ? 1 : 0, esz, cur_stream()),
+           "sinkattn_prefill");
 }
 
 void sinkattn_decode(const at::Tensor& q, const at::Tensor& kc, const at::Tensor& vc, const at::Tensor& bt, const at::Tensor& ctx,
                      int64_t Z, int64_t H, int64_t G, int64_t dim, int64_t vdim, const at::Tensor& hscale, int64_t mkind,
                      int64_t msize, bool sink, const c10::optional<at::Tensor>& gate, int64_t gate_col, at::Tensor& out,
                      const c10::optional<at::Tensor>& part, const c10::optional<at::Tensor>& pkc,
-                     const c10::optional<at::Tensor>& pvc, int64_t pool) {
+                     const c10::optional<at::Tensor>& pvc, int64_t pool, int64_t keep_first, double softcap, bool gate_elem) {
   CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(out); CHECK_LASTDIM(out);
   const int esz = esz_of(q, "q");
   const void *pkp = nullptr, *pvp = nullptr;
@@ -1513,11 +1516,12 @@ void sinkattn_decode(const at::Tensor& q, const at::Tensor& kc, const at::Tensor
     pp = part->data_ptr<float>();
   }
   long gs = 0;
-  const void* gp = gate_rows(gate, q, gate_col, H, &gs);
+  const void* gp = gate_rows(gate, q, gate_col, gate_elem ? H * vdim : H, &gs);
+  TORCH_CHECK(keep_first >= 0 && softcap >= 0, "keep_first / softcap");
   CHECK_RC(lk_sinkattn_decode(q.data_ptr(), q.stride(0), kc.data_ptr(), vc.data_ptr(), ip(bt), (int)bt.stride(0), ip(ctx), (int)B, (int)Z,
                               (int)H, (int)G, (int)dim, (int)vdim, (int)kc.size(2), fp(hscale, H, "hscale"), (int)mkind, (int)msize,
-                              sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(), out.stride(0), pp, pkp, pvp, (int)pool, esz,
-                              cur_stream()),
+                              sink ? 1 : 0, gp, gs, (int)gate_col, out.data_ptr(), out.stride(0), pp, pkp, pvp, (int)pool, (int)keep_first,
+                              (float)softcap, gate_elem ? 1 : 0, esz, cur_stream()),
            "sinkattn_decode");
 }
 
@@ -1557,7 +1561,7 @@ at::Tensor rms_cols(const at::Tensor& u, int64_t col0, int64_t n, const at::Tens
 void rot_kv_write(at::Tensor& q, int64_t H, int64_t qdim, const at::Tensor& k, int64_t G, int64_t kdim,
                   const c10::optional<at::Tensor>& kshared, int64_t sdim, const at::Tensor& v, int64_t vdim, int64_t rot_off,
                   int64_t rot, const at::Tensor& freq, double mag, const at::Tensor& positions, at::Tensor& kc, at::Tensor& vc,
-                  const at::Tensor& slots) {
+                  const at::Tensor& slots, const c10::optional<at::Tensor>& v_other, double v_blend) {
   CHECK_CUDA(q); CHECK_LASTDIM(q); CHECK_CUDA(k); CHECK_LASTDIM(k); CHECK_CUDA(v); CHECK_LASTDIM(v);
   CHECK_CUDA(slots); CHECK_I32(slots); CHECK_CONTIG(slots); CHECK_CUDA(positions); CHECK_I32(positions); CHECK_CONTIG(positions);
   const int esz = esz_of(q, "q");
@@ -1580,10 +1584,18 @@ void rot_kv_write(at::Tensor& q, int64_t H, int64_t qdim, const at::Tensor& k, i
               "caches must be K [NB, G, BS, KD], V [NB, G, VD, BS]");
   CHECK_CUDA(freq); CHECK_F32(freq); CHECK_CONTIG(freq);
   TORCH_CHECK(rot >= 0 && rot % 2 == 0 && freq.numel() >= rot / 2, "rot / freq");
+  const void* v2p = nullptr;
+  long v2s = 0;
+  if (v_other) {
+    CHECK_CUDA(*v_other); CHECK_LASTDIM(*v_other); same_type(*v_other, q, "v_other");
+    TORCH_CHECK(v_other->dim() == 2 && v_other->size(0) == T && v_other->size(1) >= G * vdim, "v_other must be [T, >= G vdim]");
+    v2p = v_other->data_ptr();
+    v2s = v_other->stride(0);
+  }
   CHECK_RC(lk_rot_kv_write(q.data_ptr(), q.stride(0), (int)H, (int)qdim, k.data_ptr(), k.stride(0), (int)G, (int)kdim, shp, shs, (int)sdim,
                            v.data_ptr(), v.stride(0), (int)vdim, (int)rot_off, (int)rot, freq.data_ptr<float>(), (float)mag,
                            ip(positions), kc.data_ptr(), vc.data_ptr(), ip(slots), (int)kc.size(2), (int)kc.size(3), (int)vc.size(2), T,
-                           esz, cur_stream()), "rot_kv_write");
+                           v2p, v2s, (float)v_blend, esz, cur_stream()), "rot_kv_write");
 }
 
 void pool_kv_write(const at::Tensor& kc, const at::Tensor& vc, at::Tensor& pkc, at::Tensor& pvc, int64_t P, const at::Tensor& bt,
@@ -1623,16 +1635,100 @@ at::Tensor gemm_grouped(const at::Tensor& x, const at::Tensor& seg, const at::Te
   return out;
 }
 
-std::vector<at::Tensor> moe_route(const at::Tensor& ids, const at::Tensor& table, int64_t E) {
-  CHECK_CUDA(ids); CHECK_I32(ids); CHECK_CONTIG(ids); CHECK_CUDA(table); CHECK_I32(table); CHECK_CONTIG(table);
+// ids absent: the table has one row per token of the step (a router's choice)
+std::vector<at::Tensor> moe_route(const c10::optional<at::Tensor>& ids, const at::Tensor& table, int64_t E) {
+  CHECK_CUDA(table); CHECK_I32(table); CHECK_CONTIG(table);
+  if (ids) { CHECK_CUDA(*ids); CHECK_I32(*ids); CHECK_CONTIG(*ids); }
   TORCH_CHECK(table.dim() == 2 && E >= 1, "table must be int32 [vocab, top]");
-  const long T = ids.numel();
+  const long T = ids ? ids->numel() : table.size(0);
   const int top = table.size(1);
-  at::Tensor seg = at::empty({E + 1}, ids.options());
-  at::Tensor order = at::empty({T * top}, ids.options());
-  CHECK_RC(lk_moe_route(ip(ids), ip(table), (int)table.size(0), top, (int)E, (int)T, seg.data_ptr<int>(), order.data_ptr<int>(),
+  at::Tensor seg = at::empty({E + 1}, table.options());
+  at::Tensor order = at::empty({T * top}, table.options());
+  CHECK_RC(lk_moe_route(ipo(ids), ip(table), (int)table.size(0), top, (int)E, (int)T, seg.data_ptr<int>(), order.data_ptr<int>(),
                         cur_stream()), "moe_route");
   return {seg, order};
+}
+
+// ---------------------------------------------------------------------------------------------
+// parallel sublayers and routed experts
+std::vector<c10::optional<at::Tensor>> stream_parallel_norm(at::Tensor& x, const c10::optional<at::Tensor>& a, const c10::optional<at::Tensor>& b,
+                                                            const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& yw,
+                                                            const c10::optional<at::Tensor>& w1, const c10::optional<at::Tensor>& w2,
+                                                            double eps, at::ScalarType out_dtype) {
+  CHECK_CUDA(x); CHECK_F32(x); CHECK_CONTIG(x);
+  TORCH_CHECK(x.dim() == 2, "x must be [T, W]");
+  TORCH_CHECK(out_dtype == at::kBFloat16 || out_dtype == at::kFloat, "out dtype");
+  const long T = x.size(0);
+  const int W = x.size(1);
+  const int esz = out_dtype == at::kFloat ? 4 : 2;
+  auto rows_of = [&](const c10::optional<at::Tensor>& t, long rows, const char* what, long* stride) -> const void* {
+    if (!t) return nullptr;
+    CHECK_CUDA(*t); CHECK_LASTDIM(*t);
+    TORCH_CHECK(t->dim() == 2 && t->size(0) == rows && t->size(1) == W, what, " must be [", rows, ", ", W, "]");
+    TORCH_CHECK(t->scalar_type() == out_dtype, what, ": dtype must be the activations'");
+    *stride = t->stride(0);
+    return t->data_ptr();
+  };
+  long as = 0, bs = 0, ys = 0;
+  const void* ap = rows_of(a, T, "a", &as);
+  const void* bp_ = rows_of(b, T, "b", &bs);
+  int top = 0;
+  const float* ywp = nullptr;
+  if (y) {
+    TORCH_CHECK(yw.has_value(), "expert rows need their weights");
+    CHECK_CUDA(*yw); CHECK_F32(*yw); CHECK_CONTIG(*yw);
+    TORCH_CHECK(yw->dim() == 2 && yw->size(0) == T && yw->size(1) >= 1, "weights must be f32 [T, top]");
+    top = yw->size(1);
+    ywp = yw->data_ptr<float>();
+  }
+  const void* yp = rows_of(y, T * std::max(top, 1), "y", &ys);
+  c10::optional<at::Tensor> o1, o2;
+  auto opt = x.options().dtype(out_dtype);
+  if (w1) o1 = at::empty({T, W}, opt);
+  if (w2) o2 = at::empty({T, W}, opt);
+  CHECK_RC(lk_stream_parallel_norm(x.data_ptr<float>(), ap, as, bp_, bs, yp, ys, ywp, top, fpo(w1, W, "norm weight 1"),
+                                   fpo(w2, W, "norm weight 2"), (float)eps, o1 ? o1->data_ptr() : nullptr, o1 ? o1->stride(0) : 0,
+                                   o2 ? o2->data_ptr() : nullptr, o2 ? o2->stride(0) : 0, T, W, esz, cur_stream()),
+           "stream_parallel_norm");
+  return {o1, o2};
+}
+
+std::vector<at::Tensor> router_topk(const at::Tensor& h, const at::Tensor& wr, int64_t top, int64_t groups, int64_t keep, double scale) {
+  CHECK_CUDA(h); CHECK_LASTDIM(h); CHECK_CUDA(wr); CHECK_F32(wr); CHECK_CONTIG(wr);
+  const int esz = esz_of(h, "h");
+  TORCH_CHECK(h.dim() == 2 && wr.dim() == 2 && wr.size(1) == h.size(1), "h [T, W], router [E, W]");
+  const long T = h.size(0);
+  at::Tensor experts = at::empty({T, top}, h.options().dtype(at::kInt));
+  at::Tensor weights = at::empty({T, top}, h.options().dtype(at::kFloat));
+  CHECK_RC(lk_router_topk(h.data_ptr(), h.stride(0), wr.data_ptr<float>(), (int)wr.size(0), (int)wr.size(1), T, (int)top, (int)groups,
+                          (int)keep, (float)scale, experts.data_ptr<int>(), weights.data_ptr<float>(), esz, cur_stream()),
+           "router_topk");
+  return {experts, weights};
+}
+
+at::Tensor clamped_glu(const at::Tensor& gu, double limit, double alpha) {
+  CHECK_CUDA(gu); CHECK_LASTDIM(gu);
+  const int esz = esz_of(gu, "gu");
+  TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0, "gu must be [T, 2F]");
+  const int F = gu.size(1) / 2;
+  at::Tensor out = at::empty({gu.size(0), F}, gu.options());
+  CHECK_RC(lk_clamped_glu(gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), gu.size(0), F, (float)limit, (float)alpha, esz,
+                          cur_stream()), "clamped_glu");
+  return out;
+}
+
+void silu_(at::Tensor& x) {
+  CHECK_CUDA(x); CHECK_LASTDIM(x);
+  TORCH_CHECK(x.dim() == 2, "x must be 2-d");
+  CHECK_RC(lk_silu_(x.data_ptr(), x.stride(0), x.size(0), (int)x.size(1), esz_of(x, "x"), cur_stream()), "silu_");
+}
+
+void sigmoid_mul_(at::Tensor& x, const at::Tensor& g) {
+  CHECK_CUDA(x); CHECK_LASTDIM(x); CHECK_CUDA(g); CHECK_LASTDIM(g);
+  same_type(g, x, "gate");
+  TORCH_CHECK(x.dim() == 2 && g.dim() == 2 && g.size(0) == x.size(0) && g.size(1) >= x.size(1), "x [T, n], gate [T, >= n]");
+  CHECK_RC(lk_sigmoid_mul_(x.data_ptr(), x.stride(0), g.data_ptr(), g.stride(0), x.size(0), (int)x.size(1), esz_of(x, "x"), cur_stream()),
+           "sigmoid_mul_");
 }
 
 at::Tensor moe_gemm(const at::Tensor& x, const at::Tensor& order, const at::Tensor& seg, const at::Tensor& w, int64_t top, bool act) {
@@ -1686,6 +1782,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("rot_kv_write", &rot_kv_write);
   m.def("pool_kv_write", &pool_kv_write);
   m.def("moe_route", &moe_route);
+  m.def("stream_parallel_norm", &stream_parallel_norm);
+  m.def("router_topk", &router_topk);
+  m.def("clamped_glu", &clamped_glu);
+  m.def("silu_", &silu_);
+  m.def("sigmoid_mul_", &sigmoid_mul_);
   m.def("gemm_grouped", &gemm_grouped);
   m.def("gemm_grouped_supported", [](int64_t N, int64_t K, bool swiglu) { return lk_gemm_grouped_supported((int)N, (int)K, swiglu ? 1 : 0) != 0; });
   m.def("moe_gemm", &moe_gemm);

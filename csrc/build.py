@@ -36,7 +36,7 @@ EXT_NAME = "_C"
 # test_ws_linear_rope_kv_matches_unfused).
 NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 NO_PACKED_FILES = ("attn_sigmoid.hip", "ssm.hip", "stream_f32.hip", "stream_ln.hip", "delta_scan.hip", "attn_sink.hip",
-                   "window_ops.hip", "moe.hip")
+                   "window_ops.hip", "moe.hip", "parallel_ops.hip")
 
 
 def _torch_paths():

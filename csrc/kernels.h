@@ -295,11 +295,11 @@ int lk_normrope_kv_write(void* qkv, long qs, long T, int H, int G, int dim, int 
 int lk_sinkattn_prefill(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* cu_q,
                         const int* ctx_lens, const int* tile_seq, const int* tile_q0, int ntiles, int H, int G, int dim, int vdim,
                         int BS, const float* hscale, int mkind, int msize, int sink, const void* gate, long gs, int gcol, void* out,
-                        long os, const void* pkc, const void* pvc, int pool, int esz, hipStream_t st);
+                        long os, const void* pkc, const void* pvc, int pool, int keep, float cap, int gelem, int esz, hipStream_t st);
 int lk_sinkattn_decode(const void* q, long qs, const void* kc, const void* vc, const int* bt, int bt_stride, const int* ctx_lens,
                        int B, int Z, int H, int G, int dim, int vdim, int BS, const float* hscale, int mkind, int msize, int sink,
                        const void* gate, long gs, int gcol, void* out, long os, float* part, const void* pkc, const void* pvc,
-                       int pool, int esz, hipStream_t st);
+                       int pool, int keep, float cap, int gelem, int esz, hipStream_t st);
 
 // csrc/window_ops.hip: gated + normed sublayer result into the f32 stream (+ the next norm), RMS norm of a column block,
 // pair rotation + key assembly + paged K / V write, pooled (mean) keys / values of finished blocks
@@ -308,10 +308,22 @@ int lk_stream_gated_norm(float* x, const void* y, long ys, int parts, const void
 int lk_rms_cols(const void* u, long us, int n, const float* w, float eps, void* out, long os, long rows, int esz, hipStream_t st);
 int lk_rot_kv_write(void* q, long qs, int H, int qdim, const void* k, long ks, int G, int kdim, const void* sh, long shs, int sdim,
                     const void* v, long vs, int vdim, int rot_off, int rot, const float* freq, float mag, const int* positions,
-                    void* kc, void* vc, const int* slots, int BS, int KD, int VD, long T, int esz, hipStream_t st);
+                    void* kc, void* vc, const int* slots, int BS, int KD, int VD, long T, const void* v2, long v2s, float blend, int esz,
+                    hipStream_t st);
 int lk_pool_kv_write(const void* kc, const void* vc, void* pkc, void* pvc, int P, const int* bt, int bt_stride, const int* ctx_lens,
                      const int* cu_q, const int* slots, int row0, int S, int max_len, int G, int BS, int dim, int vdim, int esz,
                      hipStream_t st);
+
+// csrc/parallel_ops.hip: sum of a parallel block's results into the f32 stream + the next block's two norms, f32 router with
+// group-limited top-k, clamped gated activation, element-wise silu / sigmoid gate in place
+int lk_stream_parallel_norm(float* x, const void* a, long as, const void* b, long bs, const void* y, long ys, const float* yw, int top,
+                            const float* w1, const float* w2, float eps, void* o1, long o1s, void* o2, long o2s, long rows, int W,
+                            int esz, hipStream_t st);
+int lk_router_topk(const void* h, long hs, const float* wr, int E, int W, long rows, int top, int groups, int keep, float scale,
+                   int* experts, float* weights, int esz, hipStream_t st);
+int lk_clamped_glu(const void* gu, long gs, void* out, long os, long rows, int F, float limit, float alpha, int esz, hipStream_t st);
+int lk_silu_(void* x, long xs, long rows, int n, int esz, hipStream_t st);
+int lk_sigmoid_mul_(void* x, long xs, const void* g, long gs, long rows, int n, int esz, hipStream_t st);
 
 // csrc/moe.hip: experts chosen by a table of token ids: pairs sorted by expert on the device, grouped MFMA products
 int lk_moe_route(const int* ids, const int* table, int vocab, int top, int E, int T, int* seg, int* order, hipStream_t st);

@@ -1,6 +1,7 @@
 // Feed-forward of experts chosen per token by a table of token ids (no routing network, equal weights).
 //
-//   lk_moe_route  (token, choice) pairs p = t * top + k sorted by their expert table[ids[t]][k]: seg[e] .. seg[e + 1] are
+//   lk_moe_route  (token, choice) pairs p = t * top + k sorted by their expert table[ids[t]][k] (ids null: table[t][k], the
+//                 choice a router made for each token of the step): seg[e] .. seg[e + 1] are
 //                 expert e's places in `order`.  One workgroup: a histogram and a placement with LDS atomics (the order
 //                 inside an expert's segment is arbitrary; every row of the products below is computed on its own).
 //   lk_moe_gemm   grouped product over the sorted pairs on MFMA tiles of 16 pairs: a tile's rows belong to one expert,
@@ -32,7 +33,7 @@ __global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(const int* __r
   for (int e = threadIdx.x; e < E; e += kRouteThreads) cnt[e] = 0;
   __syncthreads();
   auto expert_of = [&](int p) {
-    int id = ids[p / top];
+    int id = ids ? ids[p / top] : p / top;      // no ids: the table has one row per token of the step
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
     const int e = table[(long)id * top + p % top];
     return e < 0 ? 0 : (e >= E ? E - 1 : e);

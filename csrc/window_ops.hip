@@ -5,7 +5,8 @@
 //   lk_rms_cols           out = rms(u[:, col0 : col0 + n]) w
 //   lk_rot_kv_write       rotation of adjacent pairs by position * freq[i] (cos and sin times mag) on queries (in
 //                         place) and keys; a key head = [per-head part | part shared by the heads | zeros];
-//                         keys and values into the paged cache K [NB, G, BS, KD], V [NB, G, VD, BS]
+//                         keys and values into the paged cache K [NB, G, BS, KD], V [NB, G, VD, BS]; the cached value may
+//                         be a blend (1 - b) v + b v2 with a second set of value rows
 //   lk_pool_kv_write      mean key / value of every block of P positions whose last position is new in this step,
 //                         read from the cache (so it is the mean of what the cache holds) and filed at the block's
 //                         index b, taken as a logical position of the sequence's block table, in a second pair
@@ -155,6 +156,9 @@ struct RotParams {
   const void* v;
   long vs;
   int vdim;
+  const void* v2;   // rows of G heads of vdim columns blended into v (null: none): cached = (1 - blend) v + blend v2
+  long v2s;
+  float blend;
   int rot_off, rot;  // dimensions [rot_off, rot_off + rot) of a query / key head are rotated in adjacent pairs
   const float* freq;
   float mag;
@@ -228,11 +232,16 @@ __global__ __launch_bounds__(256) void rot_kv_write_kernel(RotParams p) {
     } else if (slot >= 0) {
       const int gh = job - p.H - p.G;
       const T* x = reinterpret_cast<const T*>(p.v) + t * p.vs + (long)gh * p.vdim;
+      const T* x2 = p.v2 ? reinterpret_cast<const T*>(p.v2) + t * p.v2s + (long)gh * p.vdim : nullptr;
       T* dst = reinterpret_cast<T*>(p.vc) + (blk * p.G + gh) * (long)p.VD * p.BS + off;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int c = lane + 64 * i;
-        if (c < p.VD) stv<T>(dst + (long)c * p.BS, c < p.vdim ? ldv<T>(x + c) : 0.f);
+        if (c < p.VD) {
+          float val = c < p.vdim ? ldv<T>(x + c) : 0.f;
+          if (x2 && c < p.vdim) val = (1.f - p.blend) * val + p.blend * ldv<T>(x2 + c);
+          stv<T>(dst + (long)c * p.BS, val);
+        }
       }
     }
   }
@@ -318,7 +327,8 @@ int lk_rms_cols(const void* u, long us, int n, const float* w, float eps, void* 
 
 int lk_rot_kv_write(void* q, long qs, int H, int qdim, const void* k, long ks, int G, int kdim, const void* sh, long shs, int sdim,
                     const void* v, long vs, int vdim, int rot_off, int rot, const float* freq, float mag, const int* positions,
-                    void* kc, void* vc, const int* slots, int BS, int KD, int VD, long T, int esz, hipStream_t st) {
+                    void* kc, void* vc, const int* slots, int BS, int KD, int VD, long T, const void* v2, long v2s, float blend, int esz,
+                    hipStream_t st) {
   if (T <= 0) return 0;
   if (H < 1 || G < 1 || qdim < 1 || kdim < 0 || sdim < 0 || (sdim > 0 && !sh) || vdim < 1 || qdim > kRotMaxHead || KD > kRotMaxHead ||
       VD > kRotMaxHead || kdim + sdim > KD || kdim + sdim < 1 || vdim > VD || rot < 0 || rot % 2 || rot_off < 0 ||
@@ -328,6 +338,7 @@ int lk_rot_kv_write(void* q, long qs, int H, int qdim, const void* k, long ks, i
   p.q = q; p.qs = qs; p.H = H; p.qdim = qdim; p.k = k; p.ks = ks; p.G = G; p.kdim = kdim; p.sh = sdim > 0 ? sh : nullptr; p.shs = shs;
   p.sdim = sdim; p.v = v; p.vs = vs; p.vdim = vdim; p.rot_off = rot_off; p.rot = rot; p.freq = freq; p.mag = mag;
   p.positions = positions; p.kc = kc; p.vc = vc; p.slots = slots; p.BS = BS; p.KD = KD; p.VD = VD;
+  p.v2 = v2; p.v2s = v2s; p.blend = blend;
   if (esz == 2) rot_kv_write_kernel<bf16_t><<<(unsigned)T, 256, 0, st>>>(p);
   else rot_kv_write_kernel<float><<<(unsigned)T, 256, 0, st>>>(p);
   LK_CHECK_LAUNCH();

@@ -129,6 +129,8 @@ class ModelPresets:
         "lebepel-1b": "lebepel-1b",
         "fusasun-tiny": "fusasun-tiny",
         "fusasun-1b": "fusasun-1b",
+        "lumedra-tiny": "lumedra-tiny",
+        "lumedra-1b": "lumedra-1b",
     })
     embedders: dict = field(default_factory=lambda: {
         "nomic-embed-text": "nomic-embed-text",

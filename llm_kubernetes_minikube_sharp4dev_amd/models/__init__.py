@@ -8,21 +8,22 @@ import torch
 
 from ..parallel.tp import SINGLE, TPGroup
 from .bert import EncoderModel
-from .configs import (DECODERS, ENCODERS, DecoderConfig, EncoderConfig, FusasunConfig, LebepelConfig, PemidraConfig, decoder_config,
+from .configs import (DECODERS, ENCODERS, DecoderConfig, EncoderConfig, FusasunConfig, LebepelConfig, LumedraConfig, PemidraConfig, decoder_config,
                       encoder_config)
 from . import llama
 from .fusasun import FusasunModel
 from .lebepel import LebepelModel
 from .llama import LlamaModel
+from .lumedra import LumedraModel
 from .opt import OPTModel
 from .pemidra import PemidraModel, ranks_from_state_dict
 
 # decoder architectures by ``cfg.arch``
 DECODER_CLASSES = {"llama": LlamaModel, "opt": OPTModel, "lebepel": LebepelModel, "pemidra": PemidraModel,
-                   "fusasun": FusasunModel}
+                   "fusasun": FusasunModel, "lumedra": LumedraModel}
 # designs with a checkpoint format of their own (config.json read by ``<Config>.from_json``, tensors by
 # ``load_state_dict_native``)
-NATIVE_CONFIGS = {"lebepel": LebepelConfig, "pemidra": PemidraConfig, "fusasun": FusasunConfig}
+NATIVE_CONFIGS = {"lebepel": LebepelConfig, "pemidra": PemidraConfig, "fusasun": FusasunConfig, "lumedra": LumedraConfig}
 
 
 def _load_safetensors_dir(path: str) -> dict:
@@ -38,7 +39,7 @@ def _load_safetensors_dir(path: str) -> dict:
 
 def build_decoder(name: str | DecoderConfig, device="cpu", dtype=torch.bfloat16, tp: TPGroup = SINGLE,
                   seed: int = 0, checkpoint: Optional[str] = None, **overrides):
-    cfg = name if isinstance(name, (DecoderConfig, LebepelConfig, PemidraConfig, FusasunConfig)) else decoder_config(name, **overrides)
+    cfg = name if isinstance(name, (DecoderConfig,) + tuple(NATIVE_CONFIGS.values())) else decoder_config(name, **overrides)
     cls = DECODER_CLASSES[cfg.arch]
     sd = _load_safetensors_dir(checkpoint) if checkpoint and cfg.arch in NATIVE_CONFIGS else None
     if sd is not None and cfg.arch == "pemidra":
@@ -119,5 +120,5 @@ def build_encoder(name: str | EncoderConfig, device="cpu", dtype=torch.bfloat16,
 
 
 __all__ = ["build_decoder", "build_encoder", "load_decoder_dir", "checkpoint_architecture", "DECODER_CLASSES",
-           "LebepelConfig", "LebepelModel", "PemidraConfig", "PemidraModel", "FusasunConfig", "FusasunModel", "NATIVE_CONFIGS", "DECODERS", "ENCODERS", "DecoderConfig", "EncoderConfig",
+           "LebepelConfig", "LebepelModel", "PemidraConfig", "PemidraModel", "FusasunConfig", "FusasunModel", "LumedraConfig", "LumedraModel", "NATIVE_CONFIGS", "DECODERS", "ENCODERS", "DecoderConfig", "EncoderConfig",
            "LlamaModel", "OPTModel", "EncoderModel"]

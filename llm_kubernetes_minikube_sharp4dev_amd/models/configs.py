@@ -234,6 +234,85 @@ class FusasunConfig:
                            for l in self.layers]}
 
 
+@dataclass
+class LumedraConfig:
+    """The Lumedra design: an f32 residual stream whose blocks run their mixer and their feed-forward side by
+    side on two norms of the same row (``x += mixer(rms(x) w1) + ff(rms(x) w2)``), three mixers in any order --
+    ``attention`` (grouped-query, no rotation, capped scores, a sliding window that keeps the first positions,
+    values blended with those of the first such layer), ``latent_attention`` (causal, element-wise output gate)
+    and ``lightning`` (decayed linear attention) -- and a feed-forward that is either dense (clamped gated
+    activation) or a mixture of experts (sigmoid router, group-limited choice, a shared expert).  The LM head is
+    the embedding table.  Every size and constant comes from the checkpoint's ``config.json``
+    (:meth:`from_json`)."""
+    name: str
+    vocab_size: int
+    hidden: int
+    layers: list                 # [HybridLayer]
+    norm_eps: float = 1e-6
+    max_position: int = 1 << 20  # nothing in the design bounds a sequence; engines pass their own limit
+    arch: str = "lumedra"
+    bos_token_id: int = 0
+    eos_token_ids: tuple = ()
+    tie_word_embeddings: bool = True
+
+    MIXERS = ("attention", "latent_attention", "lightning")
+    MLPS = ("dense", "moe")
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_json(cls, d: dict, name: str = "lumedra") -> "LumedraConfig":
+        layers = [HybridLayer(l["type"], dict(l["mixer"]), dict(l["mlp"]) if l.get("mlp") else None)
+                  for l in d["layers"]]
+        for l in layers:
+            if l.type not in cls.MIXERS:
+                raise ValueError(f"unknown mixer type {l.type!r}")
+            if l.mlp is not None and l.mlp.get("kind") not in cls.MLPS:
+                raise ValueError(f"unknown feed-forward kind {l.mlp.get('kind')!r}")
+        return cls(name=name, vocab_size=int(d["vocab"]), hidden=int(d["width"]), layers=layers,
+                   norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)), max_position=int(d.get("max_positions", 1 << 20)))
+
+    def to_json(self) -> dict:
+        return {"architecture": "Lumedra", "vocab": self.vocab_size, "width": self.hidden, "norm": {"eps": self.norm_eps},
+                "layers": [{"type": l.type, "mixer": dict(l.mixer), "mlp": dict(l.mlp) if l.mlp else None}
+                           for l in self.layers]}
+
+
+def lumedra_layers(n: int, heads: int, head_dim: int, ff: int, experts: int = 0, top: int = 2, kv_heads: Optional[int] = None,
+                   window: int = 1024, keep_first: int = 4, softcap: float = 30.0, rot_dim: int = 64, q_rank: int = 768,
+                   kv_rank: int = 512, groups: int = 4, keep: int = 2, shared_ff: int = 0, router_scale: float = 2.5,
+                   pattern=("attention", "latent_attention", "lightning"), dense_first: bool = True) -> list:
+    """``n`` layers cycling through ``pattern`` with one set of head sizes (presets and benchmarks).  ``experts``
+    0: every feed-forward is dense of size ``ff``; else experts of size ``ff`` (the first layer stays dense, of
+    ``top`` experts' size, with ``dense_first``)."""
+    kv = kv_heads or heads
+    out = []
+    for i in range(n):
+        t = pattern[i % len(pattern)]
+        if t == "attention":
+            mixer = {"heads": heads, "kv_heads": kv, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                     "softcap": softcap, "mask": {"size": window, "keep_first": keep_first}, "v_mix": True}
+        elif t == "latent_attention":
+            mixer = {"heads": heads, "dim": head_dim, "rot_dim": rot_dim, "vdim": head_dim, "q_rank": q_rank, "kv_rank": kv_rank,
+                     "scale": (head_dim + rot_dim) ** -0.5, "rot": {"base": 10000.0, "dims": rot_dim}}
+        else:
+            mixer = {"heads": heads, "dim": head_dim, "vdim": head_dim,
+                     "decay": [1.0 - 2.0 ** (-5.0 - 4.0 * j / max(heads - 1, 1)) for j in range(heads)]}
+        if not ff:
+            mlp = None
+        elif experts and not (dense_first and i == 0):
+            mlp = {"kind": "moe", "expert": {"ff": ff},
+                   "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}, "scale": router_scale}}
+            if shared_ff:
+                mlp["shared"] = {"ff": shared_ff}
+        else:
+            mlp = {"kind": "dense", "ff": ff * (top if experts else 1), "limit": 7.0}
+        out.append(HybridLayer(t, mixer, mlp))
+    return out
+
+
 def fusasun_layers(n: int, heads: int, head_dim: int, ff: int, experts: int, top: int, kv_heads: Optional[int] = None,
                    window: int = 1024, pool: int = 64, rot_dim: int = 64, q_rank: int = 768, kv_rank: int = 256,
                    pattern=("attention", "latent_attention"), original: int = 8192) -> list:
@@ -343,6 +422,15 @@ DECODERS.update({
                                 embed_scale=1.0, canon_taps=4),
 })
 
+DECODERS.update({
+    # parallel-block decoders of capped-window / latent / lightning attention with routed experts (random-init presets)
+    "lumedra-tiny": LumedraConfig("lumedra-tiny", 32768, 128, lumedra_layers(4, 4, 24, 40, 6, 2, kv_heads=2, window=20, keep_first=3,
+                                                                              softcap=15.0, rot_dim=8, q_rank=48, kv_rank=40, groups=3,
+                                                                              keep=2, shared_ff=48,
+                                                                              pattern=("attention", "latent_attention", "lightning", "attention"))),
+    "lumedra-1b": LumedraConfig("lumedra-1b", 32768, 2048, lumedra_layers(18, 16, 128, 704, 16, 4, kv_heads=4, shared_ff=1408)),
+})
+
 ENCODERS = {
     "bge-base": EncoderConfig("bge-base", "bert", 12, 768, 12, 3072, 30522, pooling="cls"),
     "minilm-l6": EncoderConfig("minilm-l6", "bert", 6, 384, 12, 1536, 30522, pooling="mean"),
@@ -370,6 +458,26 @@ def encoder_config(name: str, **overrides) -> EncoderConfig:
 
 
 def param_count(cfg) -> int:
+    if isinstance(cfg, LumedraConfig):
+        W, n = cfg.hidden, cfg.vocab_size * cfg.hidden + cfg.hidden
+        for l in cfg.layers:
+            m = l.mixer
+            if l.type == "attention":
+                n += W * (m["heads"] * (m["dim"] + m["vdim"]) + m["kv_heads"] * (m["dim"] + m["vdim"])) + 1
+            elif l.type == "latent_attention":
+                qd = m["dim"] + m["rot_dim"]
+                n += W * (m["q_rank"] + m["kv_rank"] + m["rot_dim"]) + m["q_rank"] * (1 + m["heads"] * qd) \
+                    + m["kv_rank"] * (1 + m["heads"] * (m["dim"] + m["vdim"])) + 2 * W * m["heads"] * m["vdim"]
+            else:
+                n += W * m["heads"] * (2 * m["dim"] + 3 * m["vdim"]) + m["heads"] * m["vdim"]
+            n += W
+            if l.mlp and l.mlp["kind"] == "dense":
+                n += 3 * W * l.mlp["ff"] + W
+            elif l.mlp:
+                r = l.mlp["router"]
+                n += r["experts"] * (3 * W * l.mlp["expert"]["ff"] + W) + W
+                n += 3 * W * l.mlp["shared"]["ff"] if l.mlp.get("shared") else 0
+        return n
     if isinstance(cfg, FusasunConfig):
         W, n = cfg.hidden, 2 * cfg.vocab_size * cfg.hidden + cfg.hidden
         for l in cfg.layers:

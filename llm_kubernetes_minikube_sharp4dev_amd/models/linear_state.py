@@ -1,5 +1,6 @@
-"""Linear-state mixers over the engine's per-sequence state slots: retention, the gated delta rule
-(with short causal convolutions on q, k, v) and the generalized delta rule.  All three are members of
+"""Linear-state mixers over the engine's per-sequence state slots: retention, lightning attention (retention on
+activated projections with one norm over all heads), the gated delta rule (with short causal convolutions on
+q, k, v) and the generalized delta rule.  All are members of
 
     S_t = diag(w_t) S_(t-1) - p_t (z_t^T S_(t-1)) + k_t v_t^T,    o_t = S_t^T q_t
 
@@ -81,6 +82,46 @@ def retention_mixer(h, w_in, rows: FusedRows, decay, w_out, spec: RetentionSpec,
                        meta.state_slots, meta.positions, spec.heads, spec.heads, spec.dim, spec.vdim, w_head=decay,
                        k_scale=spec.dim ** -0.5, max_len=meta.max_seq_len)
     g = ops.head_norm_gate(o, rows.cols(u, "g"), None, spec.heads, eps, ops.GATE_SILU, out_dtype)
+    return ops.linear(g, w_out)
+
+
+@dataclass
+class LightningSpec:
+    """Decayed linear attention on activated projections: q, k, v = silu of their projections, ``S <- decay_h S +
+    k v^T``, ``o = S^T q`` with no other scale; the heads' outputs are RMS-normed together over the whole row
+    with a weight, multiplied by ``sigmoid(W_g h)`` and projected."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: list = field(default_factory=list)      # one per head
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "LightningSpec":
+        s = cls(int(m["heads"]), int(m["dim"]), int(m.get("vdim", m["dim"])), [float(d) for d in m["decay"]])
+        if len(s.decay) != s.heads or not ops.delta_scan_supported(s.dim, s.vdim):
+            raise ValueError(f"unsupported lightning sizes {m}")
+        return s
+
+    def rows(self, width: int) -> FusedRows:
+        return FusedRows([("q", self.heads * self.dim), ("k", self.heads * self.dim), ("v", self.heads * self.vdim),
+                          ("g", self.heads * self.vdim)], fused_mult(width))
+
+    def make_state(self, slots: int, dtype, device):
+        return (torch.zeros(slots, self.heads, self.dim, self.vdim, dtype=torch.float32, device=device),)
+
+    def state_bytes(self, dtype) -> int:
+        return self.heads * self.dim * self.vdim * 4
+
+
+def lightning_mixer(h, w_in, rows: FusedRows, decay, norm_w, w_out, spec: LightningSpec, eps: float, state, meta, out_dtype):
+    """h [T, W] -> [T, W]: q | k | v | g in one projection, silu on the q | k | v columns in place, the decayed
+    scan (f32 state), one RMS norm over all heads times a weight times sigmoid(g), output projection."""
+    u = ops.linear(h, w_in)
+    ops.silu_(u[:, : rows.off["g"]])          # q | k | v and the zero padding between them (silu(0) = 0)
+    o = ops.delta_scan(rows.cols(u, "q"), rows.cols(u, "k"), rows.cols(u, "v"), None, None, None, state[0], meta.seq_cu,
+                       meta.state_slots, meta.positions, spec.heads, spec.heads, spec.dim, spec.vdim, w_head=decay,
+                       max_len=meta.max_seq_len)
+    g = ops.head_norm_gate(o, rows.cols(u, "g"), norm_w, 1, eps, ops.GATE_SIGMOID, out_dtype)
     return ops.linear(g, w_out)
 
 

@@ -1,5 +1,6 @@
 """Sliding-window attention mixers over the engine's paged cache: grouped-query attention whose queries
-also see one pooled (mean) key / value per block of positions that has left the window, and latent attention
+also see one pooled (mean) key / value per block of positions that has left the window, grouped-query attention
+with capped scores whose window keeps the first positions and whose values are blended across layers, and latent attention
 (queries through a normed low-rank latent, keys and values expanded from a normed latent, a rotated key segment
 common to the heads, gated heads).  Both rotate adjacent pairs of dimensions by a frequency table that carries
 the scaling rule (``RotarySpec``), and both run on the masked softmax kernels of ``ops.sink_attention_*``
@@ -132,23 +133,27 @@ class PooledWindowAttnSpec:
         return n * (2 if self.pool else 1)
 
 
-def _attend(q, k_cache, v_cache, meta: AttnMeta, H, G, dim, vdim, hscale, window, gate, gate_col, out, pool):
+def _attend(q, k_cache, v_cache, meta: AttnMeta, H, G, dim, vdim, hscale, window, gate, gate_col, out, pool, keep_first=0,
+            softcap=0.0, gate_elem=False):
+    """Prompt rows and decode rows of a step through the masked softmax kernels.  ``window`` 0: causal."""
     Tp, Bd = meta.num_prefill_tokens, meta.num_decode
+    kind = ops.MASK_WINDOW if window > 0 else ops.MASK_CAUSAL
+    opt = dict(pool=pool, keep_first=keep_first if window > 0 else 0, softcap=softcap, gate_elem=gate_elem)
     if Tp:
         if meta.sig_tiles is None and q.is_cuda:
             ts, tq = ops.sig_prefill_tiles(meta.q_lens_cpu, meta.ctx_lens_cpu)
             meta.sig_tiles = (torch.from_numpy(ts).to(q.device, non_blocking=True),
                               torch.from_numpy(tq).to(q.device, non_blocking=True))
         ops.sink_attention_prefill(q[:Tp], k_cache, v_cache, meta.block_tables_p, meta.cu_q, meta.ctx_lens_p, H, G, dim, vdim,
-                                   hscale, ops.MASK_WINDOW, window, False, gate[:Tp] if gate is not None else None, gate_col,
-                                   out[:Tp], tiles=meta.sig_tiles, pool=pool)
+                                   hscale, kind, window, False, gate[:Tp] if gate is not None else None, gate_col,
+                                   out[:Tp], tiles=meta.sig_tiles, **opt)
     if Bd:
         span = meta.block_tables_d.shape[1] * k_cache.shape[2]
-        keys = min(span, window) + (span // pool[2] if pool is not None else 0)
+        keys = (min(span, window + keep_first) if window > 0 else span) + (span // pool[2] if pool is not None else 0)
         Z = ops.sig_decode_splits(Bd, G, H // G, keys)
         ops.sink_attention_decode(q[Tp:Tp + Bd], k_cache, v_cache, meta.block_tables_d, meta.ctx_lens_d, H, G, dim, vdim,
-                                  hscale, ops.MASK_WINDOW, window, False, gate[Tp:Tp + Bd] if gate is not None else None,
-                                  gate_col, out[Tp:Tp + Bd], splits=Z, pool=pool)
+                                  hscale, kind, window, False, gate[Tp:Tp + Bd] if gate is not None else None,
+                                  gate_col, out[Tp:Tp + Bd], splits=Z, **opt)
     return out
 
 
@@ -179,11 +184,68 @@ def pooled_window_attention(qkv: torch.Tensor, caches, meta: AttnMeta, spec: Poo
 
 
 @dataclass
+class CappedWindowAttnSpec:
+    """Grouped-query softmax attention without rotation: scores ``cap * tanh(scale q.k / cap)`` (``softcap`` 0:
+    plain), query i sees j <= i with ``i - j < window`` or ``j < keep_first`` (``window`` 0: causal).  With
+    ``v_mix`` the cached value is ``(1 - lambda) v + lambda v_first``, ``v_first`` the values that the model's
+    first such layer projects for the same token (that layer itself caches its own).  Head sizes here are the
+    kernels' (multiples of 8); the checkpoint's may be smaller (zero weight rows / columns)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0
+    keep_first: int = 0
+    softcap: float = 0.0
+    v_mix: bool = False
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "CappedWindowAttnSpec":
+        mask = m.get("mask") or {}
+        s = cls(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m.get("vdim", m["dim"])),
+                float(m.get("scale", int(m["dim"]) ** -0.5)), int(mask.get("size", 0)), int(mask.get("keep_first") or 0),
+                float(m.get("softcap") or 0.0), bool(m.get("v_mix", False)))
+        if s.heads % s.kv_heads or s.window < 0 or s.keep_first < 0 or s.softcap < 0:
+            raise ValueError(f"unsupported attention sizes {m}")
+        return s
+
+    def padded(self) -> "CappedWindowAttnSpec":
+        return CappedWindowAttnSpec(self.heads, self.kv_heads, _pad8(self.dim), _pad8(self.vdim), self.scale, self.window,
+                                    self.keep_first, self.softcap, self.v_mix)
+
+    def make_caches(self, num_blocks: int, block_size: int, dtype, device) -> tuple:
+        return _cache_pair(num_blocks, self.kv_heads, block_size, self.dim, self.vdim, dtype, device)
+
+    def bytes_per_token(self, dtype) -> int:
+        return self.kv_heads * (self.dim + self.vdim) * torch.tensor([], dtype=dtype).element_size()
+
+
+def capped_window_attention(qkv: torch.Tensor, caches, meta: AttnMeta, spec: CappedWindowAttnSpec, hscale, freq, v_first=None,
+                            v_blend: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """qkv [T, q | k | v] straight from the fused projection (``spec``: the padded sizes).  One kernel files k and
+    the (blended) v in the paged cache; then prompt rows and decode rows attend through the cache.  ``v_first``
+    [T, G vdim]: the values to blend in with weight ``v_blend``.  ``freq``: an unused frequency table (nothing
+    is rotated).  [T, H vdim]."""
+    H, G, dim, vdim = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+    T = qkv.shape[0]
+    if out is None:
+        out = torch.empty(T, H * vdim, dtype=qkv.dtype, device=qkv.device)
+    k_cache, v_cache = caches[0], caches[1]
+    kcol, vcol = H * dim, (H + G) * dim
+    ops.rot_kv_write(qkv, H, dim, qkv[:, kcol:], G, dim, None, 0, qkv[:, vcol:], vdim, 0, 0, freq, 1.0, meta.positions, k_cache, v_cache,
+                     meta.slots, v_other=v_first, v_blend=v_blend)
+    return _attend(qkv, k_cache, v_cache, meta, H, G, dim, vdim, hscale, spec.window, None, 0, out, None, spec.keep_first,
+                   spec.softcap)
+
+
+@dataclass
 class LatentAttnSpec:
     """Latent attention: ``c_q = rms(W_dq h) w_q``, ``q = W_uq c_q`` (per head ``dim`` plain and ``rot_dim``
     rotated columns); ``W_dkv h`` = ``kv_rank`` latent columns (normed: c) and ``rot_dim`` columns of one
     rotated key segment common to the heads; per head key ``[W_uk c | common segment]``, value ``W_uv c``; sliding
-    window; each head's output times ``sigmoid(W_g h)``.  The cache holds the expanded keys and values
+    window (``window`` 0: causal); the output times ``sigmoid(W_g h)``, one gate per head or (``gate_elem``) one
+    per output element.  The cache holds the expanded keys and values
     (``heads`` key / value heads): a sliding window bounds what a decoded token reads, and scores against
     the latent would cost ``kv_rank / dim`` times the products."""
     heads: int
@@ -195,17 +257,24 @@ class LatentAttnSpec:
     scale: float
     window: int
     rot: RotarySpec = field(default_factory=RotarySpec)
+    gate_elem: bool = False
 
     @classmethod
-    def from_dict(cls, m: dict) -> "LatentAttnSpec":
+    def from_dict(cls, m: dict, gate_elem: bool = False, causal_ok: bool = False) -> "LatentAttnSpec":
         mask, rd = m.get("mask") or {}, int(m.get("rot_dim", 0))
         rot = dict(m.get("rot") or {})
         rot["dims"] = rd
         s = cls(int(m["heads"]), int(m["dim"]), rd, int(m.get("vdim", m["dim"])), int(m["q_rank"]), int(m["kv_rank"]),
-                float(m.get("scale", (int(m["dim"]) + rd) ** -0.5)), int(mask.get("size", 0)), RotarySpec.from_dict(rot, "ramp"))
-        if s.window < 1 or rd % 2:
+                float(m.get("scale", (int(m["dim"]) + rd) ** -0.5)), int(mask.get("size", 0)), RotarySpec.from_dict(rot, "ramp"),
+                gate_elem)
+        if s.window < (0 if causal_ok else 1) or rd % 2:
             raise ValueError(f"unsupported latent attention sizes {m}")
         return s
+
+    @property
+    def gate_cols(self) -> int:
+        """Columns of the gate projection: one per head, or one per (padded) output element."""
+        return self.heads * self.vdim_p if self.gate_elem else self.heads
 
     @property
     def kdim(self) -> int:
@@ -240,4 +309,5 @@ def latent_window_attention(u, rows, uv_col: int, w_uq, w_ukv, dq_norm, dkv_norm
     k_cache, v_cache = caches[0], caches[1]
     ops.rot_kv_write(q, H, kd, kv, H, dim, u[:, rows.off["dkv"] + spec.kv_rank:], rd, kv[:, uv_col:], vd, dim, rd, freq,
                      spec.rot.magnitude, meta.positions, k_cache, v_cache, meta.slots)
-    return _attend(q, k_cache, v_cache, meta, H, H, kd, vd, hscale, spec.window, u, rows.off["g"], out, None)
+    return _attend(q, k_cache, v_cache, meta, H, H, kd, vd, hscale, spec.window, u, rows.off["g"], out, None,
+                   gate_elem=spec.gate_elem)

@@ -20,7 +20,8 @@ from .mixers import (conv_silu, embed_pos, gated_group_rmsnorm, linear_swiglu_an
                      softcap, ssm_scan, stream_rmsnorm, unitnorm_kv_write, embed_stream, stream_layernorm, gelu_tanh_mul,
                      dual_rmsnorm_mean, normrope_kv_write, sink_attention_prefill, sink_attention_decode, mask_first_key,
                      pooled_blocks_seen, MASK_CAUSAL, MASK_CHUNK, MASK_WINDOW)
-from .window import moe_route, pool_kv_write, rms_cols, rot_kv_write, stream_gated_norm, table_experts  # noqa: F401
+from .window import moe_route, pool_kv_write, rms_cols, rot_kv_write, run_experts, stream_gated_norm, table_experts  # noqa: F401
+from .routed import clamped_glu, routed_experts, router_topk, sigmoid_mul_, silu_, stream_parallel_norm  # noqa: F401
 from .delta import (delta_scan, delta_scan_supported, gated_delta_prep, general_delta_prep, head_norm_gate, tanh_,  # noqa: F401
                     GATE_SIGMOID, GATE_SILU)
 

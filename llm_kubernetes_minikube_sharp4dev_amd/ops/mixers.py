@@ -397,13 +397,16 @@ def pooled_blocks_seen(qpos, mask_size: int, pool: int):
     return max(0, qpos - mask_size + 1) // pool
 
 
-def _sink_rows(q, k, v, qpos, hscale, mask_kind, mask_size, sink, pooled=None):
+def _sink_rows(q, k, v, qpos, hscale, mask_kind, mask_size, sink, pooled=None, keep_first=0, cap=0.0):
     """q f32 [S, H, dim] at positions qpos [S]; k/v f32 [n, G, *] at positions 0..n-1.  ``pooled`` = (pk, pv
     f32 [nb, G, *], pool): one more key / value per block of ``pool`` positions, seen by a query once the
-    block is entirely behind its window, in the same softmax."""
+    block is entirely behind its window, in the same softmax.  ``keep_first``: the first positions stay
+    visible behind a window; ``cap`` > 0: scores become cap * tanh(score / cap)."""
     H, G = q.shape[1], k.shape[1]
     rep = H // G
     s = torch.einsum("ihd,jhd->hij", q, k.repeat_interleave(rep, dim=1)) * hscale.view(-1, 1, 1)
+    if cap > 0:
+        s = cap * torch.tanh(s / cap)
     j = torch.arange(k.shape[0], device=q.device).view(1, -1)
     i = qpos.view(-1, 1)
     if pooled is not None and pooled[0].shape[0]:
@@ -427,7 +430,7 @@ def _sink_rows(q, k, v, qpos, hscale, mask_kind, mask_size, sink, pooled=None):
         lo = (i - mask_size + 1).clamp(min=0)
     else:
         lo = torch.zeros_like(i)
-    seen = (j <= i) & (j >= lo)
+    seen = (j <= i) & ((j >= lo) | (j < keep_first))
     s = s.masked_fill(~seen[None], float("-inf"))
     m = s.amax(-1, keepdim=True)
     if sink:
@@ -450,9 +453,25 @@ def _pooled_of(pool, table, n):
     return pk, pv, P
 
 
+def _check_mask_options(mask_kind, pool, keep_first):
+    if pool is not None and mask_kind != MASK_WINDOW:
+        raise ValueError("pooled blocks go with a sliding window")
+    if keep_first and (mask_kind != MASK_WINDOW or pool is not None):
+        raise ValueError("kept first positions go with a sliding window without pooled blocks")
+
+
+def _gated(o, gate, r0, r1, gate_col, H, vdim, gate_elem):
+    """o f32 [S, H, vdim] times the sigmoid of the gate rows [r0, r1): one column per head, or per element."""
+    if gate is None:
+        return o
+    if gate_elem:
+        return o * torch.sigmoid(gate[r0:r1, gate_col:gate_col + H * vdim].float()).view(-1, H, vdim)
+    return o * torch.sigmoid(gate[r0:r1, gate_col:gate_col + H].float()).unsqueeze(-1)
+
+
 def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H: int, G: int, dim: int, vdim: int, hscale,
                            mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, tiles=None, q_lens_cpu=None,
-                           pool=None):
+                           pool=None, keep_first: int = 0, softcap: float = 0.0, gate_elem: bool = False):
     """Softmax attention of query chunks over their sequences' cached keys inside the mask
     (``mask_first_key``), with ``sink``: one more term of score 0 and no value in the denominator.
     ``hscale`` f32 [H]: the score multiplier of each head.  ``gate`` (or None): rows aligned with ``q``
@@ -460,9 +479,11 @@ def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H:
     its sigmoid.  q: rows whose first H * dim columns are the prepared queries; out [T, H * vdim].
     ``pool`` = (pooled K cache, pooled V cache, P), window masks only: beside its window a query sees one
     pooled key / value per block of P positions entirely behind the window (``pooled_blocks_seen``), filed by
-    ``pool_kv_write`` at the logical position b of the same block table."""
-    if pool is not None and mask_kind != MASK_WINDOW:
-        raise ValueError("pooled blocks go with a sliding window")
+    ``pool_kv_write`` at the logical position b of the same block table.
+    ``keep_first`` (window masks, no pooling): positions below it stay visible to every later query.  ``softcap`` >
+    0: a score s becomes softcap * tanh(s / softcap) before the softmax.  ``gate_elem``: the gate has one column
+    per output element, ``gate_col + h * vdim + d``, instead of one per head."""
+    _check_mask_options(mask_kind, pool, keep_first)
     if use_hip(q):
         if tiles is None:
             ql = q_lens_cpu if q_lens_cpu is not None else (cu_q[1:] - cu_q[:-1]).tolist()
@@ -470,7 +491,8 @@ def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H:
             tiles = (torch.from_numpy(ts).to(q.device), torch.from_numpy(tq).to(q.device))
         pk, pv, P = pool if pool is not None else (None, None, 0)
         lib().sinkattn_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, tiles[0], tiles[1], H, G, dim, vdim, hscale,
-                               int(mask_kind), int(mask_size), bool(sink), gate, int(gate_col), out, pk, pv, int(P))
+                               int(mask_kind), int(mask_size), bool(sink), gate, int(gate_col), out, pk, pv, int(P),
+                               int(keep_first), float(softcap), bool(gate_elem))
         return out
     cu = cu_q.tolist()
     for b in range(len(cu) - 1):
@@ -479,35 +501,31 @@ def sink_attention_prefill(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, H:
         k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
         qq = q[s0:s1, : H * dim].float().view(s1 - s0, H, dim)
         qpos = torch.arange(n - (s1 - s0), n, device=q.device)
-        o = _sink_rows(qq, k, v, qpos, hscale, mask_kind, mask_size, sink, _pooled_of(pool, block_tables[b], n))
-        if gate is not None:
-            o = o * torch.sigmoid(gate[s0:s1, gate_col:gate_col + H].float()).unsqueeze(-1)
-        out[s0:s1, : H * vdim] = o.reshape(s1 - s0, H * vdim).to(out.dtype)
+        o = _sink_rows(qq, k, v, qpos, hscale, mask_kind, mask_size, sink, _pooled_of(pool, block_tables[b], n), keep_first, softcap)
+        out[s0:s1, : H * vdim] = _gated(o, gate, s0, s1, gate_col, H, vdim, gate_elem).reshape(s1 - s0, H * vdim).to(out.dtype)
     return out
 
 
 def sink_attention_decode(q, k_cache, v_cache, block_tables, ctx_lens, H: int, G: int, dim: int, vdim: int, hscale,
                           mask_kind: int, mask_size: int, sink: bool, gate, gate_col: int, out, splits: int = 1, part=None,
-                          pool=None):
+                          pool=None, keep_first: int = 0, softcap: float = 0.0, gate_elem: bool = False):
     """One query row per sequence at its last position (ctx - 1) over its cached keys inside the mask
     (and the pooled blocks before it: see ``sink_attention_prefill``)."""
     B = q.shape[0]
-    if pool is not None and mask_kind != MASK_WINDOW:
-        raise ValueError("pooled blocks go with a sliding window")
+    _check_mask_options(mask_kind, pool, keep_first)
     if use_hip(q):
         if splits > 1 and part is None:
             part = torch.empty(B * H * splits * (vdim + 2), dtype=torch.float32, device=q.device)
         pk, pv, P = pool if pool is not None else (None, None, 0)
         lib().sinkattn_decode(q, k_cache, v_cache, block_tables, ctx_lens, int(splits), H, G, dim, vdim, hscale, int(mask_kind),
-                              int(mask_size), bool(sink), gate, int(gate_col), out, part, pk, pv, int(P))
+                              int(mask_size), bool(sink), gate, int(gate_col), out, part, pk, pv, int(P), int(keep_first),
+                              float(softcap), bool(gate_elem))
         return out
     for b in range(B):
         n = int(ctx_lens[b])
         k, v = _gather_kv(k_cache, v_cache, block_tables[b], n)
         qq = q[b:b + 1, : H * dim].float().view(1, H, dim)
         o = _sink_rows(qq, k, v, torch.tensor([n - 1], device=q.device), hscale, mask_kind, mask_size, sink,
-                       _pooled_of(pool, block_tables[b], n))
-        if gate is not None:
-            o = o * torch.sigmoid(gate[b:b + 1, gate_col:gate_col + H].float()).unsqueeze(-1)
-        out[b:b + 1, : H * vdim] = o.reshape(1, H * vdim).to(out.dtype)
+                       _pooled_of(pool, block_tables[b], n), keep_first, softcap)
+        out[b:b + 1, : H * vdim] = _gated(o, gate, b, b + 1, gate_col, H, vdim, gate_elem).reshape(1, H * vdim).to(out.dtype)
     return out

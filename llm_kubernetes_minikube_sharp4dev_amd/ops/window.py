@@ -24,7 +24,7 @@ from ._ext import lib, use_hip
 # from this many (token, choice) pairs per expert on average the experts run on the dense GEMM's 256-row tiles
 GROUPED_DENSE_MIN_ROWS = 128
 
-__all__ = ["stream_gated_norm", "rms_cols", "rot_kv_write", "pool_kv_write", "table_experts", "moe_route"]
+__all__ = ["stream_gated_norm", "rms_cols", "rot_kv_write", "pool_kv_write", "table_experts", "run_experts", "moe_route"]
 
 
 def stream_gated_norm(x, y, g, g_bias, w_post, w_next, eps: float, out_dtype=torch.bfloat16, parts: int = 1):
@@ -54,17 +54,19 @@ def rms_cols(u, col0: int, n: int, w, eps: float):
 
 
 def rot_kv_write(q, H: int, qdim: int, k, G: int, kdim: int, kshared, sdim: int, v, vdim: int, rot_off: int, rot: int, freq,
-                 mag: float, positions, k_cache, v_cache, slots):
+                 mag: float, positions, k_cache, v_cache, slots, v_other=None, v_blend: float = 0.0):
     """Rotate and file one step's queries and keys.
 
     ``q`` rows hold H heads of ``qdim`` columns (rotated in place); a key head is ``[k head part (kdim) |
     kshared (sdim, the same for all G heads) | zeros]`` up to the cache's head size; ``v`` rows hold G heads
     of ``vdim`` columns.  Dimensions ``rot_off + 2 i`` and ``rot_off + 2 i + 1`` (i < rot / 2) of every query and
     key head are rotated by the angle ``position * freq[i]`` (f32), cos and sin both times ``mag``.  Keys and values
-    go to the paged cache at ``slots`` (< 0: nothing is cached)."""
+    go to the paged cache at ``slots`` (< 0: nothing is cached).  With ``v_other`` (rows of G heads of ``vdim``
+    columns, e.g. an earlier layer's values of the same tokens) the cached value is the f32 blend
+    ``(1 - v_blend) * v + v_blend * v_other``."""
     if use_hip(q):
         lib().rot_kv_write(q, H, qdim, k, G, kdim, kshared, sdim, v, vdim, int(rot_off), int(rot), freq, float(mag), positions,
-                           k_cache, v_cache, slots)
+                           k_cache, v_cache, slots, v_other, float(v_blend))
         return q
     T = q.shape[0]
     half = rot // 2
@@ -89,6 +91,8 @@ def rot_kv_write(q, H: int, qdim: int, k, G: int, kdim: int, kshared, sdim: int,
         kk = rot(kk)
     vv = torch.zeros(T, G, v_cache.shape[2], dtype=torch.float32, device=q.device)
     vv[..., :vdim] = v[:, : G * vdim].float().reshape(T, G, vdim)
+    if v_other is not None:
+        vv[..., :vdim] = (1.0 - v_blend) * vv[..., :vdim] + v_blend * v_other[:, : G * vdim].float().reshape(T, G, vdim)
     BS = k_cache.shape[2]
     sl = slots[:T].long()
     ok = sl >= 0
@@ -128,11 +132,12 @@ def pool_kv_write(k_cache, v_cache, pk_cache, pv_cache, P: int, block_tables, ct
 
 def moe_route(ids, table, experts: int):
     """(seg int32 [experts + 1], order int32 [T * top]): the (token, choice) pairs ``t * top + k`` sorted by
-    their expert ``table[ids[t], k]``; pairs ``order[seg[e] : seg[e + 1]]`` belong to expert e."""
-    if use_hip(ids):
+    their expert ``table[ids[t], k]`` (``ids`` None: ``table[t, k]``, a table with one row per token of the
+    step); pairs ``order[seg[e] : seg[e + 1]]`` belong to expert e."""
+    if use_hip(table):
         seg, order = lib().moe_route(ids, table, int(experts))
         return seg, order
-    e = table[ids.long()].reshape(-1).long()
+    e = (table if ids is None else table[ids.long()]).reshape(-1).long()
     order = torch.sort(e, stable=True).indices.to(torch.int32)
     seg = torch.zeros(experts + 1, dtype=torch.int32)
     seg[1:] = torch.cumsum(torch.bincount(e, minlength=experts), 0)
@@ -145,6 +150,12 @@ def table_experts(h, ids, table, w_gate_up, w_down, top: int):
     padded with zero rows to ffp), ``w_down`` [E, W, ffp].  Returns the experts' results un-summed,
     [T * top, W] in h's dtype with a token's ``top`` rows adjacent: the consumer averages them in f32
     (``stream_gated_norm(parts=top)``)."""
+    return run_experts(h, ids, table, w_gate_up, w_down, top)
+
+
+def run_experts(h, ids, table, w_gate_up, w_down, top: int):
+    """The expert products behind ``table_experts`` (``ids`` int32 [T] index the table's rows) and
+    ``routed_experts`` (``ids`` None: ``table`` int32 [T, top] holds each row's own choice)."""
     T, W = h.shape
     E, ffp = w_gate_up.shape[0], w_down.shape[2]
     if use_hip(h):
@@ -157,7 +168,7 @@ def table_experts(h, ids, table, w_gate_up, w_down, top: int):
             return lib().gemm_grouped(mid, seg, w_down, False, None, order)
         mid = lib().moe_gemm(h, order, seg, w_gate_up, int(top), True)          # [T * top, ffp], sorted-pair order
         return lib().moe_gemm(mid, order, seg, w_down, int(top), False)         # [T * top, W], pair order
-    e = table[ids.long()].long()                                                # [T, top]
+    e = (table if ids is None else table[ids.long()]).long()                    # [T, top]
     out = torch.zeros(T * top, W, dtype=h.dtype, device=h.device)
     pair_e = e.reshape(-1)
     rows = torch.arange(T * top, device=h.device) // top
