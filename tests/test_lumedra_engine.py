@@ -1,0 +1,368 @@
+"""The Lumedra decoder through the framework's engine (model registry, loader, runner, paged cache, state
+slots, scheduler, hipGraph decode, replay and generation entry points) against the plain float64 forward
+of ``lumedra_oracle``.  Small random models of several shapes; CPU path and (``gpu`` marker) HIP kernels
+in f32 and bf16."""
+import io
+import json
+
+import pytest
+import torch
+
+import lumedra_oracle as O
+from llm_kubernetes_minikube_sharp4dev_amd.engine.llm_engine import LLMEngine
+from llm_kubernetes_minikube_sharp4dev_amd.engine.sampling import SamplingParams
+from llm_kubernetes_minikube_sharp4dev_amd.models import LumedraConfig, LumedraModel, build_decoder, load_decoder_dir
+
+CPU32 = pytest.param("cpu", torch.float32, id="cpu-f32")
+GPU32 = pytest.param("cuda", torch.float32, id="gpu-f32", marks=pytest.mark.gpu)
+GPU16 = pytest.param("cuda", torch.bfloat16, id="gpu-bf16", marks=pytest.mark.gpu)
+ALL = [CPU32, GPU32, GPU16]
+
+
+def att(heads, kv, dim, vdim, scale, size=None, keep=0, cap=0.0, v_mix=False):
+    m = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": scale, "v_mix": v_mix}
+    if size is not None:
+        m["mask"] = {"size": size, "keep_first": keep}
+    if cap:
+        m["softcap"] = cap
+    return {"type": "attention", "mixer": m}
+
+
+def lat(heads, dim, rd, vdim, qr, kvr, scale, base):
+    return {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "rot_dim": rd, "vdim": vdim, "q_rank": qr, "kv_rank": kvr,
+                                                  "scale": scale, "rot": {"base": base, "dims": rd}}}
+
+
+def lig(heads, dim, vdim, decay):
+    return {"type": "lightning", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "decay": decay}}
+
+
+def dense(layer, ff, limit):
+    return dict(layer, mlp={"kind": "dense", "ff": ff, "limit": limit})
+
+
+def moe(layer, ff, experts, top, groups=None, keep=None, scale=1.0, shared=0):
+    r = {"experts": experts, "top": top, "scale": scale}
+    if groups:
+        r["groups"] = {"count": groups, "keep": keep}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": r}
+    if shared:
+        mlp["shared"] = {"ff": shared}
+    return dict(layer, mlp=mlp)
+
+
+def bare(layer):
+    return dict(layer, mlp=None)
+
+
+def config(layers, width, vocab=97, eps=1e-5):
+    return {"architecture": "Lumedra", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": layers}
+
+
+CONFIGS = {
+    # all three mixers; GQA 2:1 with a window of 20 that keeps 3 first positions (neither a page's size), capped scores, two
+    # layers that blend values (the second blends the first's in); dense and routed feed-forwards, groups of 2 of which 2 of 3
+    # are kept, a shared expert
+    "tri": config([dense(att(4, 2, 24, 16, 0.25, 20, 3, 8.0, True), 40, 1.2),
+                   moe(lat(3, 12, 8, 20, 24, 20, 0.3, 40.0), 20, 6, 2, 3, 2, 1.5, 24),
+                   moe(lig(3, 8, 12, [0.7, 0.93, 0.995]), 20, 6, 2, 3, 2, 1.5, 24),
+                   moe(att(4, 2, 24, 16, 0.25, 20, 3, 8.0, True), 20, 6, 3, 2, 2, 0.8)], 48),
+    # the lightning mixer first and without a feed-forward; one head everywhere; one expert of one; a window of 7 that keeps
+    # nothing, no cap, no blending; then a layer that would blend but is the only one (keeps its own), keep_first = window;
+    # every expert chosen; sizes that are multiples of nothing convenient
+    "odd": config([bare(lig(1, 10, 14, [0.9])),
+                   moe(lat(1, 10, 6, 14, 9, 11, 0.4, 100.0), 13, 1, 1),
+                   dense(att(1, 1, 10, 14, 0.3, 7), 11, 0.7),
+                   moe(att(3, 3, 10, 6, 0.3, 5, 5, 50.0, True), 13, 4, 4, 2, 2, 2.0, 9)], 36, vocab=61, eps=1e-6),
+    # causal attention without a window (capped), a window longer than any test sequence, more kept positions than the window is
+    # long, wide heads, groups of ONE expert (a group's score is its only score), top = what the kept groups hold
+    "wide": config([moe(att(2, 1, 72, 40, 0.1, None, 0, 5.0, True), 24, 4, 2, 4, 2, 1.0),
+                    dense(lig(2, 72, 40, [0.98, 0.6]), 50, 3.0),
+                    dense(lat(2, 72, 40, 48, 40, 56, 0.1, 10000.0), 24, 0.9),
+                    moe(att(2, 1, 72, 40, 0.15, 4096, 2, 0.0, True), 24, 3, 1, shared=16),
+                    dense(att(2, 2, 40, 72, 0.15, 9, 14), 24, 2.0)], 56, vocab=130),
+    # projections the MFMA / weight-streaming kernels tile: no vendor GEMM, decode steps captured in hipGraphs
+    "mid": config([moe(att(4, 2, 64, 64, 0.125, 48, 4, 20.0, True), 128, 8, 2, 4, 2, 1.5, 128),
+                   moe(lat(4, 64, 32, 64, 256, 256, 0.1, 10000.0), 128, 8, 2, 4, 2, 1.5, 128),
+                   moe(lig(4, 64, 64, [0.9, 0.95, 0.99, 0.999]), 128, 8, 2, 4, 2, 1.5, 128),
+                   dense(att(4, 2, 64, 64, 0.125, 48, 4, 20.0, True), 256, 4.0)], 256, vocab=768),
+}
+_models = {}
+
+
+def model_and_weights(name, device, dtype, seed=3):
+    key = (name, device, dtype)
+    if key not in _models:
+        m = build_decoder(LumedraConfig.from_json(CONFIGS[name], name), device=device, dtype=dtype, seed=seed)
+        _models[key] = (m, {k: v.cpu() for k, v in m.native_state_dict().items()})
+    return _models[key]
+
+
+def engine(m, tokens=512, seqs=4, **kw):
+    return LLMEngine(m, None, block_size=16, max_model_len=tokens, max_num_seqs=seqs, num_blocks=-(-tokens // 16), eos_ids=set(), **kw)
+
+
+def toks(n, vocab, seed):
+    return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def close(got, want, dtype):
+    """Largest error of a position over the vocabulary, relative to the largest logit: f32 runs within 1e-4 at
+    every position; bf16 runs (weights rounded alike on both sides, activations rounded by the framework only)
+    within 3e-2 at half of the positions and 0.15 at all."""
+    want = want.double()
+    err = (got.double().cpu() - want).abs().reshape(want.shape[0], -1).amax(1) / want.abs().max()
+    if dtype == torch.float32:
+        return float(err.max()) < 1e-4, float(err.max())
+    return float(err.median()) < 3e-2 and float(err.max()) < 0.15, (float(err.median()), float(err.max()))
+
+
+def replay(eng, rid, tokens, cuts, end=True):
+    """Feed ``tokens`` in portions of the sizes ``cuts`` (the rest one by one); logits of every position."""
+    out, at = [], 0
+    sizes = list(cuts)
+    while at < len(tokens):
+        n = min(sizes.pop(0) if sizes else 1, len(tokens) - at)
+        last = at + n == len(tokens)
+        out.append(eng.replay_step([(rid, tokens[at:at + n], list(range(n)))], [rid] if last and end else []))
+        at += n
+    return torch.cat(out)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_prompt_streams_and_logits(name, device, dtype):
+    m, sd = model_and_weights(name, device, dtype)
+    t = toks(45, m.cfg.vocab_size, 1)
+    want, streams = O.forward(CONFIGS[name], sd, t, True)
+    eng = engine(m)
+    from llm_kubernetes_minikube_sharp4dev_amd.engine.sequence import Sequence
+    sq = Sequence(list(t), SamplingParams(max_tokens=1))
+    assert eng.scheduler.admit_forced(sq, len(t))
+    si, _ = eng.runner.prepare([(sq, 0, len(t))], want={id(sq): list(range(len(t)))})
+    ids, meta = eng.runner._meta(si)
+    taps = []
+    with torch.inference_mode():
+        m(ids, meta, eng.runner.kv_caches, taps=taps)
+    eng.scheduler.finish(sq, "stop")
+    assert len(taps) == len(streams) == m.cfg.num_layers
+    for r, (a, b) in enumerate(zip(taps, streams)):     # the f32 stream after every layer
+        ok, err = close(a, b, dtype)
+        assert ok, (r, err)
+    ok, err = close(replay(eng, "w", t, [len(t)]), want, dtype)
+    assert ok, err
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("name", ["tri", "odd"])
+def test_prefill_equals_token_by_token_and_portions(name, device, dtype):
+    """One step for the whole prompt, one token per step, and portions of changing size down to two tokens
+    (cut inside pages and windows, and between the kept first positions) give the same logits at every position."""
+    m, sd = model_and_weights(name, device, dtype)
+    t = toks(70, m.cfg.vocab_size, 2)
+    want = O.forward(CONFIGS[name], sd, t)
+    eng = engine(m)
+    for cuts in ([70], [], [1, 2, 2, 3, 16, 17, 5, 2], [33, 2, 31], [2, 7, 8]):
+        ok, err = close(replay(eng, "r", t, cuts), want, dtype)
+        assert ok, (cuts, err)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_mixed_batches_equal_each_request_alone(device, dtype):
+    """Five requests of unequal lengths share steps: portions of some beside single tokens of others, a
+    request sitting out steps, requests ending and a new one taking the freed pages and slot."""
+    name = "tri"
+    m, sd = model_and_weights(name, device, dtype)
+    V = m.cfg.vocab_size
+    T = {"a": toks(60, V, 10), "b": toks(21, V, 11), "c": toks(9, V, 12), "d": toks(40, V, 13), "e": toks(33, V, 14)}
+    want = {k: O.forward(CONFIGS[name], sd, v) for k, v in T.items()}
+    plan = [[("a", 17)], [("a", 15), ("b", 20), ("c", 1)], [("a", 1), ("b", 1), ("c", 2), ("d", 31)],
+            [("a", 1), ("c", 6), ("d", 1)], [("a", 26), ("d", 1)], [("d", 7), ("e", 2)], [("e", 30)], [("e", 1)]]
+    eng = engine(m, tokens=160, seqs=4)   # a + b + c + d live together need 64 + 32 + 16 + 48 tokens of pages
+    at = {k: 0 for k in T}
+    got = {k: [] for k in T}
+    for step in plan:
+        entries, end = [], []
+        for k, n in step:
+            entries.append((k, T[k][at[k]:at[k] + n], list(range(n))))
+            at[k] += n
+            if at[k] == len(T[k]):
+                end.append(k)
+        lg = eng.replay_step(entries, end)
+        r = 0
+        for k, n in step:
+            got[k].append(lg[r:r + n])
+            r += n
+    assert at == {k: len(v) for k, v in T.items()}
+    assert eng.allocator.num_free == eng.runner.num_blocks and eng.state_pool.num_free == 4
+    for k in T:
+        ok, err = close(torch.cat(got[k]), want[k], dtype)
+        assert ok, (k, err)
+        # the same portions alone, in the same number format: nothing but rounding may separate the two runs
+        alone = replay(eng, k + "-alone", T[k], [n for step in plan for kk, n in step if kk == k])
+        d = float((alone.double() - torch.cat(got[k]).double()).abs().max() / want[k].abs().max())
+        assert d < (1e-5 if dtype == torch.float32 else 6e-2), (k, d)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_freed_pages_and_slots_are_used_again(device, dtype):
+    """A pool of exactly one request's size and ONE state slot: every request runs in the pages and the slot
+    (the lightning state of a longer predecessor) its predecessor left, and repeats its own first run bit for
+    bit; a second live request is refused."""
+    m, sd = model_and_weights("odd", device, dtype)
+    V = m.cfg.vocab_size
+    a, b = toks(41, V, 20), toks(48, V, 21)
+    eng = engine(m, tokens=48, seqs=1)
+    first = replay(eng, "a", a, [20, 5])
+    other = replay(eng, "b", b, [3, 30])
+    again = replay(eng, "a2", a, [20, 5])
+    assert torch.equal(first, again)
+    assert close(first, O.forward(CONFIGS["odd"], sd, a), dtype)[0]
+    assert close(other, O.forward(CONFIGS["odd"], sd, b), dtype)[0]
+    eng.replay_step([("x", a[:5], [])])
+    with pytest.raises(RuntimeError):
+        eng.replay_step([("y", b[:5], [])])
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_long_decode_through_pages_and_windows(device, dtype):
+    """150 single-token steps after a short prompt (across many page borders, far past the window, the kept
+    first positions still seen), two requests side by side."""
+    m, sd = model_and_weights("tri", device, dtype)
+    V = m.cfg.vocab_size
+    a, b = toks(170, V, 30), toks(152, V, 31)
+    eng = engine(m, tokens=352, seqs=2)
+    ga, gb = [eng.replay_step([("a", a[:20], list(range(20)))])], [eng.replay_step([("b", b[:2], list(range(2)))])]
+    for i in range(150):
+        lg = eng.replay_step([("a", [a[20 + i]], [0]), ("b", [b[2 + i]], [0])])
+        ga.append(lg[:1])
+        gb.append(lg[1:])
+    for got, t in ((ga, a), (gb, b)):
+        ok, err = close(torch.cat(got), O.forward(CONFIGS["tri"], sd, t), dtype)
+        assert ok, err
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("name", ["tri", "wide"])
+def test_greedy_generation_through_the_scheduler(name, device, dtype):
+    """``LLMEngine.generate``: the scheduler admits, chunks (a 24-token step budget) and batches three
+    prompts; every generated token must be the oracle's argmax for its prefix (or within a near tie)."""
+    m, sd = model_and_weights(name, device, dtype)
+    V = m.cfg.vocab_size
+    prompts = [toks(50, V, 40), toks(7, V, 41), toks(1, V, 42)]
+    eng = LLMEngine(m, None, block_size=16, max_model_len=256, max_num_seqs=3, num_blocks=16, eos_ids=set(),
+                    max_num_batched_tokens=24)
+    seqs = eng.generate(prompts, SamplingParams.greedy(12))
+    assert eng.allocator.num_free == 16 and eng.state_pool.num_free == 3
+    for p, s in zip(prompts, seqs):
+        assert len(s.output_ids) == 12
+        full = p + list(s.output_ids)
+        lg = O.forward(CONFIGS[name], sd, full[:-1])[len(p) - 1:]
+        for i, tid in enumerate(s.output_ids):
+            gap = float(lg[i].max() - lg[i, tid])
+            assert gap <= (1e-3 if dtype == torch.float32 else 0.25) * float(lg[i].max() - lg[i].min()), (i, gap)
+
+
+def test_checkpoint_directory_selects_the_model_and_replays(tmp_path):
+    """config.json + model.safetensors on disk: the registry picks the class by the architecture name, the
+    loader checks shapes, and the trace command writes the logits it is asked for."""
+    import numpy as np
+    from safetensors.torch import save_file
+
+    from llm_kubernetes_minikube_sharp4dev_amd.engine.replay import run_trace
+
+    m, sd = model_and_weights("odd", "cpu", torch.float32)
+    cfg = CONFIGS["odd"]
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps(cfg))
+    sd16 = {k: v.to(torch.bfloat16) for k, v in sd.items()}
+    save_file(sd16, str(d / "model.safetensors"))
+    m2 = load_decoder_dir(str(d), dtype=torch.float32)
+    assert isinstance(m2, LumedraModel) and m2.cfg.num_layers == 4 and m2.cfg.norm_eps == 1e-6
+    assert m2.layers[0].kind is None and m2.layers[1].mlp.top == 1 and m2.layers[3].mlp.keep == 2 and m2.layers[3].mix.spec.keep_first == 5
+    assert "l2.mix.vmix" not in m2.native_state_dict()          # a layer that does not blend has no such tensor
+    t = toks(30, 61, 50)
+    want = O.forward(cfg, sd16, t)
+    steps = [{"step": 0, "entries": [{"id": "q", "tokens": t[:19], "want": [0, 18]}], "end": []},
+             {"step": 1, "entries": [{"id": "q", "tokens": t[19:20], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "q", "tokens": t[20:], "want": [9]}, {"id": "p", "tokens": t[:4], "want": [3]}],
+              "end": ["q", "p"]}]
+    out = io.StringIO()
+    assert run_trace(str(d), "float32", str(tmp_path / "o"), 64, lines=[json.dumps(s) for s in steps], out=out, device="cpu") == 0
+    assert out.getvalue().split() == ["done", "0", "done", "1", "done", "2"]
+    l0 = torch.from_numpy(np.fromfile(tmp_path / "o" / "0.f32", dtype="<f4")).view(2, 61)
+    l2 = torch.from_numpy(np.fromfile(tmp_path / "o" / "2.f32", dtype="<f4")).view(2, 61)
+    assert not (tmp_path / "o" / "1.f32").exists()
+    assert close(l0, want[[0, 18]], torch.float32)[0] and close(l2, want[[29, 3]], torch.float32)[0]
+    bad = dict(sd16)
+    bad["l2.mix.q"] = bad["l2.mix.q"][:-1]
+    with pytest.raises(ValueError):
+        LumedraModel(m2.cfg, dtype=torch.float32).load_state_dict_native(bad)
+    bad = dict(sd16)
+    bad["l3.mlp.router"] = bad["l3.mlp.router"][:-1]             # fewer rows than the layer has experts
+    with pytest.raises(ValueError):
+        LumedraModel(m2.cfg, dtype=torch.float32).load_state_dict_native(bad)
+
+
+def test_config_round_trip_and_refusals():
+    cfg = LumedraConfig.from_json(CONFIGS["tri"])
+    assert cfg.to_json()["layers"] == CONFIGS["tri"]["layers"] and cfg.tie_word_embeddings
+    bad = json.loads(json.dumps(CONFIGS["tri"]))
+    bad["layers"][0]["type"] = "convolution"
+    with pytest.raises(ValueError):
+        LumedraConfig.from_json(bad)
+    bad = json.loads(json.dumps(CONFIGS["tri"]))
+    bad["layers"][1]["mlp"]["router"]["top"] = 5                  # more than the kept groups hold
+    with pytest.raises(ValueError):
+        build_decoder(LumedraConfig.from_json(bad), device="cpu", dtype=torch.float32)
+    bad = json.loads(json.dumps(CONFIGS["tri"]))
+    bad["layers"][3]["mixer"]["vdim"] = 24                        # blending layers must agree on their values' shape
+    with pytest.raises(ValueError):
+        build_decoder(LumedraConfig.from_json(bad), device="cpu", dtype=torch.float32)
+
+
+@pytest.mark.gpu
+def test_captured_decode_graph_matches_the_oracle():
+    """bf16 on the GPU with sizes the framework's own GEMM kernels tile: decode steps replay a captured
+    hipGraph (state slots and block tables in its static buffers, router and experts on the device); prompt
+    portions, then 60 single tokens (past a window's end) for two requests that start at different times,
+    against the float64 forward."""
+    m, sd = model_and_weights("mid", "cuda", torch.bfloat16)
+    V = m.cfg.vocab_size
+    a, b = toks(110, V, 60), toks(95, V, 61)
+    wa, wb = O.forward(CONFIGS["mid"], sd, a), O.forward(CONFIGS["mid"], sd, b)
+    eng = engine(m, tokens=256, seqs=2)
+    ga = [eng.replay_step([("a", a[:33], list(range(33)))]), eng.replay_step([("a", a[33:50], list(range(17)))])]
+    gb = []
+    for i in range(60):
+        entries = [("a", [a[50 + i]], [0])]
+        if i == 5:
+            entries.append(("b", b[:35], list(range(35))))
+        elif i > 5:
+            entries.append(("b", [b[35 + i - 6]], [0]))
+        lg = eng.replay_step(entries)
+        ga.append(lg[:1])
+        if i >= 5:
+            gb.append(lg[1:])
+    captured = [k for k, st in eng.runner.graphs.items() if st.get("graph") is not None]
+    assert captured, "no decode bucket was captured"
+    for got, want, n in ((ga, wa, 110), (gb, wb, 35 + 54)):
+        ok, err = close(torch.cat(got), want[:n], torch.bfloat16)
+        assert ok, err
+
+
+def test_served_through_the_model_manager(tmp_path):
+    """The serving stack's model manager builds the preset, wraps it in an engine with state slots and
+    prefix caching off, and generates through the server's pipelined step loop."""
+    import asyncio
+
+    from llm_kubernetes_minikube_sharp4dev_amd.config import Config
+    from llm_kubernetes_minikube_sharp4dev_amd.serving.model_manager import ModelManager
+
+    cfg = Config()
+    cfg.engine.dtype, cfg.engine.max_num_seqs, cfg.engine.max_model_len = "float32", 4, 256
+    mgr = ModelManager(cfg, device="cpu", engine_overrides={"num_blocks": 32})
+    h = mgr.generator("lumedra-tiny")
+    eng = h.engine
+    assert isinstance(eng.model, LumedraModel) and eng.state_pool.num_slots == 4 and not eng.allocator.prefix_caching

@@ -1,0 +1,314 @@
+"""The Lumedra decoder's mechanisms, each alone, against the plain float64 implementations of
+``lumedra_oracle``: the framework's mixers over a paged cache / state slots, whole sequences, cut into
+portions and decoded token by token, on the CPU path and (``gpu`` marker) on the HIP kernels in f32 and
+bf16.  Where random weights would hide a fault (a window's edge, the last kept position, a far key, a group
+that shuts a high score out) the weights and inputs are made so that it shows."""
+import math
+
+import pytest
+import torch
+
+import lumedra_oracle as O
+from llm_kubernetes_minikube_sharp4dev_amd import ops
+from llm_kubernetes_minikube_sharp4dev_amd.models import LumedraConfig, build_decoder
+from test_fusasun_mixers import q16, rel_err, rnd, step_meta, tol
+
+CPU32 = pytest.param("cpu", torch.float32, id="cpu-f32")
+GPU32 = pytest.param("cuda", torch.float32, id="gpu-f32", marks=pytest.mark.gpu)
+GPU16 = pytest.param("cuda", torch.bfloat16, id="gpu-bf16", marks=pytest.mark.gpu)
+ALL = [CPU32, GPU32, GPU16]
+BS = 16
+EPS = 1e-5
+
+
+def one_layer(kind, mixer, W, device, dtype, seed=5, sd=None):
+    """A one-layer model of the mechanism (random weights through the checkpoint names, or ``sd``) and its tensors."""
+    cfg = LumedraConfig.from_json({"architecture": "Lumedra", "vocab": 11, "width": W, "norm": {"eps": EPS},
+                                   "layers": [{"type": kind, "mixer": mixer, "mlp": None}]})
+    m = build_decoder(cfg, device=device, dtype=dtype, seed=seed)
+    if sd is not None:
+        full = {k: v.cpu() for k, v in m.native_state_dict().items()}
+        full.update(sd)
+        m.load_state_dict_native(full)
+    out = {k[len("l0.mix."):]: v.cpu().double() for k, v in m.native_state_dict().items() if k.startswith("l0.mix.")}
+    return m, out
+
+
+def run_mixer(m, h, cuts, device, dtype, slot=1, nblocks=40, caches=None):
+    """The layer's mixer over ``h`` [T, W] fed in portions of the sizes ``cuts`` (the rest as decode rows)."""
+    T = h.shape[0]
+    blocks = list(range(nblocks - 1, nblocks - 1 - (T + BS - 1) // BS, -1))   # pages in descending order
+    caches = caches or m.make_caches(nblocks, BS, 3)
+    out, at, sizes = [], 0, list(cuts)
+    while at < T:
+        dec = not sizes
+        n = 1 if dec else min(sizes.pop(0), T - at)
+        meta = step_meta([(at, n, blocks, slot, dec)], device)
+        with torch.inference_mode():
+            y = m._mixer(m.layers[0], h[at:at + n].to(dtype).to(device).contiguous(), meta, caches[0], {})
+        out.append(y.float().cpu())
+        at += n
+    return torch.cat(out)
+
+
+def want_mixer(kind, h, mixer, w):
+    if kind == "attention":
+        return O.window_attention(h, mixer, w)[0]
+    if kind == "latent_attention":
+        return O.latent_attention(h, mixer, w, EPS)
+    return O.lightning(h, mixer, w, EPS)
+
+
+ATT = {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 16, "scale": 0.3, "softcap": 6.0, "mask": {"size": 13, "keep_first": 4}, "v_mix": False}
+LAT = {"heads": 3, "dim": 12, "rot_dim": 6, "vdim": 20, "q_rank": 14, "kv_rank": 18, "scale": 0.35, "rot": {"dims": 6, "base": 30.0}}
+LIG = {"heads": 3, "dim": 10, "vdim": 12, "decay": [0.5, 0.9, 0.999]}
+KINDS = {"attention": ATT, "latent_attention": LAT, "lightning": LIG}
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("kind", list(KINDS))
+def test_mixer_whole_tokenwise_and_portions(kind, device, dtype):
+    """A whole prompt, one token per step, and portions down to two tokens (then decode rows) over pages handed
+    out in descending order, all into caches and state slots that hold another sequence's leftovers."""
+    W = 40
+    m, w = one_layer(kind, KINDS[kind], W, device, dtype)
+    g = torch.Generator().manual_seed(1)
+    h = q16(rnd(g, 53, W))
+    want = want_mixer(kind, h, KINDS[kind], w)
+    for cuts in ([53], [], [2, 3, 16, 2, 11, 5], [31, 2]):
+        caches = m.make_caches(40, BS, 3)
+        for c in caches[0]:
+            c.copy_(torch.randn(c.shape, generator=g).to(c.dtype))       # finite leftovers, never NaN
+        got = run_mixer(m, h, cuts, device, dtype, caches=caches)
+        assert rel_err(got, want) < tol(dtype), (cuts, rel_err(got, want))
+
+
+def copy_attention(size, keep, cap, H=2, d=8, dv=8):
+    """An attention layer whose projections copy input columns (q | k | v side by side, the output projection
+    the heads' values), so that a test writes queries, keys and values directly."""
+    W = H * d + d + dv
+    mixer = {"heads": H, "kv_heads": 1, "dim": d, "vdim": dv, "scale": 1.0, "v_mix": False}
+    if size:
+        mixer["mask"] = {"size": size, "keep_first": keep}
+    if cap:
+        mixer["softcap"] = cap
+    eye = torch.eye(W, dtype=torch.float64)
+    o = torch.zeros(W, H * dv, dtype=torch.float64)
+    o[:H * dv] = torch.eye(H * dv, dtype=torch.float64)
+    sd = {"l0.mix.q": eye[:H * d], "l0.mix.k": eye[H * d:H * d + d], "l0.mix.v": eye[H * d + d:], "l0.mix.o": o}
+    return W, mixer, {k: v.float() for k, v in sd.items()}
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("size,keep,cap,star", [(13, 4, 6.0, 3), (13, 4, 6.0, 4), (16, 1, 0.0, 0), (16, 1, 0.0, 1), (32, 0, 9.0, 0),
+                                               (7, 9, 5.0, 8), (7, 9, 5.0, 9), (20, 16, 0.0, 15), (20, 17, 7.0, 16)])
+def test_window_edge_and_last_kept_position(size, keep, cap, star, device, dtype):
+    """One key made to stand out at position ``star``: every query sees its marker while the key is inside its
+    window or among the kept first positions, and loses it on the very position the mask says -- in a whole
+    prompt, token by token, and with portions cut at the window's edge."""
+    H, d, dv, T = 2, 8, 8, 75
+    W, mixer, sd = copy_attention(size, keep, cap)
+    m, w = one_layer("attention", mixer, W, device, dtype, sd=sd)
+    h = torch.zeros(T, W, dtype=torch.float64)
+    h[:, 0] = 1.0
+    h[:, d] = 1.0                                         # both heads' queries: e_0
+    h[star, H * d] = 12.0                                 # the key that stands out (score 12, or the cap)
+    h[star, H * d + d + 2] = 1.0                          # its value: the marker in dimension 2
+    want = O.window_attention(h, mixer, w)[0]
+    seen = torch.tensor([star <= i and (i - star < size or star < keep) for i in range(T)])
+    assert bool((want[seen, 2] > 0.5).all()) and bool((want[~seen, 2].abs() < 1e-9).all()) and 0 < int(seen.sum())
+    for cuts in ([T], [], [star + size - 1, 2, 2], [star + 1, size - 1, 3]):
+        got = run_mixer(m, h, [c for c in cuts if c > 0], device, dtype)
+        assert rel_err(got, want) < tol(dtype), (cuts, rel_err(got, want))
+        assert bool((got[seen, 2] > 0.5).all()) and bool((got[~seen, 2].abs() < 1e-3).all()), cuts
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("size,keep", [(None, 0), (64, 2), (300, 0)])
+def test_far_key_among_hundreds(size, keep, device, dtype):
+    """A key 400 positions back (second page of the sequence), reachable by the causal mask, the kept first
+    positions, or not at all: prompt in two portions, then decode rows over many pages."""
+    H, d, dv, T, star = 2, 8, 8, 420, 1
+    W, mixer, sd = copy_attention(size, keep, 0.0)
+    m, w = one_layer("attention", mixer, W, device, dtype, sd=sd)
+    g = torch.Generator().manual_seed(3)
+    h = q16(rnd(g, T, W, scale=0.3))
+    h[:, :H * d] = 0.0
+    h[:, 0] = 1.0
+    h[:, d] = 1.0
+    h[star, H * d] = 14.0
+    h[star, H * d + d:] = 0.0
+    h[star, H * d + d + 5] = 40.0
+    want = O.window_attention(h, mixer, w)[0]
+    far = want[400:, 5]
+    assert bool((far > 20).all()) if (size is None or keep > star) else bool((far.abs() < 5).all())
+    got = run_mixer(m, h, [200, 190], device, dtype)
+    assert rel_err(got, want) < tol(dtype), rel_err(got, want)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_lightning_long_state_and_slot_reuse(device, dtype):
+    """300 tokens through the recurrent state (a decay close to one keeps the first tokens alive): whole, in
+    portions and token by token; then another sequence takes the same slot and must start from zero."""
+    W = 32
+    mixer = {"heads": 2, "dim": 16, "vdim": 24, "decay": [0.9995, 0.8]}
+    m, w = one_layer("lightning", mixer, W, device, dtype)
+    g = torch.Generator().manual_seed(7)
+    h, h2 = q16(rnd(g, 300, W)), q16(rnd(g, 37, W))
+    want, want2 = O.lightning(h, mixer, w, EPS), O.lightning(h2, mixer, w, EPS)
+    caches = m.make_caches(40, BS, 3)
+    for cuts in ([300], [7, 2, 130, 100], [250]):
+        assert rel_err(run_mixer(m, h, cuts, device, dtype, caches=caches), want) < tol(dtype), cuts
+        assert rel_err(run_mixer(m, h2, [20], device, dtype, caches=caches), want2) < tol(dtype), cuts
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_value_blend_in_the_cache_write(device, dtype):
+    H, G, d, dv, T = 2, 2, 8, 8, 5
+    g = torch.Generator().manual_seed(2)
+    qkv = q16(rnd(g, T, (H + G) * d + G * dv)).to(dtype).to(device)
+    other = q16(rnd(g, T, G * dv)).to(dtype).to(device)
+    kc = torch.zeros(2, G, BS, d, dtype=dtype, device=device)
+    vc = torch.zeros(2, G, dv, BS, dtype=dtype, device=device)
+    slots = torch.tensor([17, 3, 31, -1, 0], dtype=torch.int32, device=device)
+    pos = torch.arange(T, dtype=torch.int32, device=device)
+    freq = torch.zeros(1, device=device)
+    ops.rot_kv_write(qkv, H, d, qkv[:, H * d:], G, d, None, 0, qkv[:, (H + G) * d:], dv, 0, 0, freq, 1.0, pos, kc, vc, slots,
+                     v_other=other, v_blend=0.3)
+    want = 0.7 * qkv[:, (H + G) * d:].double() + 0.3 * other.double()
+    for t, s in enumerate(slots.tolist()):
+        if s >= 0:
+            assert rel_err(vc[s // BS, :, :, s % BS].reshape(-1), want[t].cpu()) < tol(dtype)
+            assert torch.equal(kc[s // BS, :, s % BS].reshape(-1), qkv[t, H * d:(H + G) * d])
+    assert int((vc.abs().sum(dim=(1, 2)) > 0).sum()) == 4       # the row without a slot cached nothing
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("E,groups,keep,top", [(16, 4, 3, 2), (6, 3, 2, 2), (4, 4, 2, 2), (8, 1, 1, 3), (5, 1, 1, 5), (64, 8, 4, 8), (1, 1, 1, 1),
+                                              (12, 2, 1, 6)])
+def test_router_against_the_oracle(E, groups, keep, top, device, dtype):
+    g = torch.Generator().manual_seed(E)
+    W, T = 24, 37
+    h = q16(rnd(g, T, W))
+    wr = q16(rnd(g, E, W, scale=0.5))
+    r = {"experts": E, "top": top, "scale": 1.7}
+    if groups > 1:
+        r["groups"] = {"count": groups, "keep": keep}
+    ex, wt = ops.router_topk(h.to(dtype).to(device), wr.float().to(device), top, groups, keep, 1.7)
+    assert ex.dtype == torch.int32 and wt.dtype == torch.float32
+    z = h @ wr.T
+    for t in range(T):
+        chosen, wgt = O.route(z[t], r)
+        got = dict(zip(ex[t].tolist(), wt[t].tolist()))
+        assert sorted(got) == sorted(chosen), t
+        for e, a in zip(chosen, wgt.tolist()):
+            assert abs(got[e] - a) < 1e-5 * 1.7, (t, e)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_router_groups_shut_a_high_score_out(device, dtype):
+    """The largest score of all sits alone in a weak group: with 2 of 3 groups kept it cannot be chosen."""
+    s = torch.tensor([0.9, 0.1, 0.1, 0.1, 0.6, 0.58, 0.2, 0.2, 0.55, 0.54, 0.3, 0.1], dtype=torch.float64)
+    wr = torch.zeros(12, 8, dtype=torch.float64)
+    wr[:, 0] = torch.log(s / (1 - s))
+    h = torch.zeros(3, 8, dtype=torch.float64)
+    h[:, 0] = 1.0
+    ex, wt = ops.router_topk(h.to(dtype).to(device), wr.float().to(device), 3, 3, 2, 1.0)
+    assert sorted(ex[0].tolist()) == [4, 5, 8]
+    assert abs(float(wt[0].sum()) - 1.0) < 1e-5
+    ex, _ = ops.router_topk(h.to(dtype).to(device), wr.float().to(device), 3, 1, 1, 1.0)     # no groups: the 0.9 is first
+    assert sorted(ex[1].tolist()) == [0, 4, 5]
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("W,top", [(36, 1), (256, 2), (1000, 3), (1024, 2), (2050, 2)])
+def test_stream_update_with_both_norms(W, top, device, dtype):
+    g = torch.Generator().manual_seed(W)
+    T = 9
+    x0, a, b = rnd(g, T, W, scale=3.0).float(), q16(rnd(g, T, W)), q16(rnd(g, T, W))
+    y, yw = q16(rnd(g, T * top, W)), rnd(g, T, top).abs().float()
+    w1, w2 = rnd(g, W).float() + 1.0, rnd(g, W).float() + 1.0
+    dev = lambda t: t.to(device) if t.dtype == torch.float32 else t.to(dtype).to(device)   # noqa: E731
+    for use in ((1, 1, 1), (1, 0, 0), (0, 1, 1), (0, 0, 0)):
+        x = x0.clone().to(device)
+        h1, h2 = ops.stream_parallel_norm(x, dev(a) if use[0] else None, dev(b) if use[1] else None, dev(y) if use[2] else None,
+                                          dev(yw) if use[2] else None, dev(w1), dev(w2), EPS, dtype)
+        want = x0.double() + use[0] * a + use[1] * b + use[2] * (y.view(T, top, W) * yw.double().view(T, top, 1)).sum(1)
+        assert rel_err(x, want) < 1e-6
+        n = want / torch.sqrt((want * want).mean(-1, keepdim=True) + EPS)
+        assert rel_err(h1, n * w1.double()) < tol(dtype) and rel_err(h2, n * w2.double()) < tol(dtype)
+    x = x0.clone().to(device)
+    assert ops.stream_parallel_norm(x, dev(a), None, None, None, None, None, EPS, dtype) == (None, None)
+    assert rel_err(x, x0.double() + a) < 1e-6
+    h1, h2 = ops.stream_parallel_norm(x, None, None, None, None, dev(w1), None, EPS, dtype)
+    assert h2 is None and h1.shape == (T, W)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_clamped_gated_activation_and_elementwise_ops(device, dtype):
+    g = torch.Generator().manual_seed(4)
+    gu = q16(rnd(g, 7, 2 * 52, scale=3.0))
+    got = ops.clamped_glu(gu.to(dtype).to(device), 1.5, 1.702)
+    gg, uu = gu[:, :52].clamp(max=1.5), gu[:, 52:].clamp(-1.5, 1.5)
+    assert rel_err(got, gg * O.sigmoid(1.702 * gg) * (uu + 1)) < tol(dtype)
+    assert float(got.float().max()) <= 1.5 * 2.5 + 0.05            # both clamps bound the result
+    x = q16(rnd(g, 5, 40))
+    buf = x.to(dtype).to(device).clone()
+    ops.silu_(buf[:, 8:32])
+    assert rel_err(buf[:, 8:32], O.silu(x[:, 8:32])) < tol(dtype) and torch.equal(buf[:, :8].cpu().double(), x[:, :8])
+    buf = x.to(dtype).to(device).clone()
+    ops.sigmoid_mul_(buf[:, :16], buf[:, 16:32])
+    assert rel_err(buf[:, :16], x[:, :16] * O.sigmoid(x[:, 16:32])) < tol(dtype)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+@pytest.mark.parametrize("T,W,ff,E,top", [(11, 40, 24, 5, 2), (3, 36, 13, 1, 1), (70, 64, 32, 4, 3), (600, 256, 128, 4, 2)])
+def test_routed_experts_against_plain_products(T, W, ff, E, top, device, dtype):
+    """Chosen experts' feed-forwards, un-summed: sizes the vector loads do and do not divide, one expert, and a
+    step large enough for the grouped form of the dense GEMM (bf16 on the GPU)."""
+    g = torch.Generator().manual_seed(T)
+    ffp = -(-ff // 8) * 8
+    h = q16(rnd(g, T, W))
+    gate_up, down = torch.zeros(E, 2 * ffp, W, dtype=torch.float64), torch.zeros(E, W, ffp, dtype=torch.float64)
+    gate_up[:, :ff], gate_up[:, ffp:ffp + ff] = q16(rnd(g, E, ff, W, scale=W ** -0.5)), q16(rnd(g, E, ff, W, scale=W ** -0.5))
+    down[:, :, :ff] = q16(rnd(g, E, W, ff, scale=ff ** -0.5))
+    choice = torch.rand(T, E, generator=g).argsort(1)[:, :top].to(torch.int32)
+    got = ops.routed_experts(h.to(dtype).to(device), choice.to(device), gate_up.to(dtype).to(device), down.to(dtype).to(device))
+    want = torch.zeros(T * top, W, dtype=torch.float64)
+    for t in range(T):
+        for k in range(top):
+            e = int(choice[t, k])
+            mid = O.silu(h[t] @ gate_up[e, :ff].T) * (h[t] @ gate_up[e, ffp:ffp + ff].T)
+            want[t * top + k] = mid @ down[e, :, :ff].T
+    assert rel_err(got, want) < tol(dtype), rel_err(got, want)
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
+def test_latent_far_key_and_gate(device, dtype):
+    """Causal latent attention over 300 positions (every position attends the first ones across many pages),
+    whole against portions + decode rows; the element gate closes single output columns."""
+    W = 40
+    m, w = one_layer("latent_attention", LAT, W, device, dtype, seed=9)
+    g = torch.Generator().manual_seed(11)
+    h = q16(rnd(g, 300, W))
+    want = O.latent_attention(h, LAT, w, EPS)
+    assert rel_err(run_mixer(m, h, [150, 2, 120], device, dtype), want) < tol(dtype)
+    sd = {"l0.mix.g": torch.zeros_like(w["g"]).float()}
+    sd["l0.mix.g"][5] = -200.0 * torch.sign(torch.ones(W))          # a gate row that is shut whenever sum(h) > 0
+    m2, w2 = one_layer("latent_attention", LAT, W, device, dtype, seed=9, sd=sd)
+    hp = h[:40].abs()
+    want2 = O.latent_attention(hp, LAT, w2, EPS)
+    got2 = run_mixer(m2, hp, [17], device, dtype)
+    assert rel_err(got2, want2) < tol(dtype)
+
+
+def test_decay_and_cap_constants_reach_the_mixers():
+    """Values a config may make equal or 1 elsewhere: different decays per head, a cap below the scores, a scale of one."""
+    cfg = LumedraConfig.from_json({"architecture": "Lumedra", "vocab": 11, "width": 16, "norm": {"eps": EPS},
+                                   "layers": [{"type": "lightning", "mixer": dict(LIG), "mlp": None},
+                                              {"type": "attention", "mixer": dict(ATT, scale=1.0), "mlp": None}]})
+    m = build_decoder(cfg, device="cpu", dtype=torch.float32)
+    assert [round(float(v), 6) for v in m.layers[0].mix.decay] == [0.5, 0.9, 0.999]
+    s = m.layers[1].mix.spec
+    assert (s.softcap, s.window, s.keep_first, s.scale) == (6.0, 13, 4, 1.0) and float(m.layers[1].mix.hscale[0]) == 1.0
+    assert math.isclose(m.layers[1].mix.blend, 0.0)
