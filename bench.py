@@ -142,7 +142,7 @@ def parse():
     ap.add_argument("--json-out", default=None)
     ap.add_argument("--decoder-bench", action="store_true",
                     help="instead of the headline workload: prefill and decode tokens/s of the hybrid decoders "
-                         "(Lebepel by default; -- --models pemidra,lebepel,llama or fusasun,llama for the others) beside a Llama decoder of "
+                         "(Lebepel by default; -- --models pemidra,lebepel,llama, fusasun,llama or lumedra,fusasun,llama for the others) beside a Llama decoder of "
                          "equal size at a few layer sizes (benchmarks/decoder_bench.py; its own options follow after --)")
     args, rest = ap.parse_known_args()
     if rest and not args.decoder_bench:

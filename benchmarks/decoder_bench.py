@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Prefill and decode throughput of the hybrid decoders (Lebepel; Pemidra with ``--models pemidra,lebepel``;
-Fusasun with ``--models fusasun,llama``) beside a Llama decoder of the same width, depth, heads, head size, feed-forward and vocabulary (random
+Fusasun with ``--models fusasun,llama``; Lumedra with ``--models lumedra,fusasun,llama``) beside a Llama decoder of the same width, depth, heads, head size, feed-forward and vocabulary (random
 weights, bf16, one GPU), all through the same engine: prefill = S fresh prompts of L tokens in one step, decode = B sequences at
 context C, one token each per step (hipGraph replay).  ``bench.py --decoder-bench`` runs this.
 
@@ -32,8 +32,9 @@ VOCAB = 32768
 
 def models(width: int, which: str, device):
     from llm_kubernetes_minikube_sharp4dev_amd.models import build_decoder
-    from llm_kubernetes_minikube_sharp4dev_amd.models.configs import (FusasunConfig, LebepelConfig, PemidraConfig, decoder_config,
-                                                                      fusasun_layers, lebepel_layers, pemidra_layers)
+    from llm_kubernetes_minikube_sharp4dev_amd.models.configs import (FusasunConfig, LebepelConfig, LumedraConfig, PemidraConfig,
+                                                                      decoder_config, fusasun_layers, lebepel_layers, lumedra_layers,
+                                                                      pemidra_layers)
 
     L, H, G, D, FF, sh, sp, sn, sg = SIZES[width]
     if which == "lebepel":
@@ -51,6 +52,15 @@ def models(width: int, which: str, device):
         cfg = FusasunConfig(f"fusasun-w{width}", VOCAB, width,
                             fusasun_layers(L, H, D, FF // 2, 16, 2, kv_heads=G, window=512, pool=64, rot_dim=64,
                                            q_rank=max(512, width // 2), kv_rank=512), embed_scale=1.0, canon_taps=4)
+    elif which == "lumedra":
+        # capped-window attention (window 512 + 4 kept positions, values blended), causal latent attention (latent 512 + 64
+        # rotated) and lightning attention in turn, the same heads and head size; the first feed-forward dense, the others 16
+        # experts of a quarter of it in 4 groups (2 kept), two per token, beside a shared expert of half of it: the products a
+        # token runs are those of the dense model
+        cfg = LumedraConfig(f"lumedra-w{width}", VOCAB, width,
+                            lumedra_layers(L, H, D, FF // 4, 16, 2, kv_heads=G, window=512, keep_first=4, rot_dim=64,
+                                           q_rank=max(512, width // 2), kv_rank=512, groups=4, keep=2, shared_ff=FF // 2))
+        cfg.layers[0].mlp["ff"] = FF
     else:
         cfg = decoder_config("llama-3-8b", num_layers=L, hidden=width, num_heads=H, num_kv_heads=G, head_dim=D,
                              intermediate=FF, vocab_size=VOCAB, max_position=8192)
@@ -107,7 +117,7 @@ def run(width: int, which: str, a) -> dict:
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--sizes", default="1024,2048,4096")
-    ap.add_argument("--models", default="lebepel,llama", help="comma list of lebepel, pemidra, fusasun, llama")
+    ap.add_argument("--models", default="lebepel,llama", help="comma list of lebepel, pemidra, fusasun, lumedra, llama")
     ap.add_argument("--prefill-seqs", type=int, default=4)
     ap.add_argument("--prefill-len", type=int, default=1024)
     ap.add_argument("--decode-batch", type=int, default=64)
