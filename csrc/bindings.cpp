@@ -1346,7 +1346,7 @@ const float* f32_rows(const c10::optional<at::Tensor>& t, long T, long n, const 
 at::Tensor delta_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& w,
                       const c10::optional<at::Tensor>& p, const c10::optional<at::Tensor>& z, at::Tensor& state, const at::Tensor& cu,
                       const at::Tensor& slots, const at::Tensor& positions, int64_t H, int64_t Hk, int64_t dk, int64_t dv,
-                      const c10::optional<at::Tensor>& w_head, double k_scale, int64_t max_len, int64_t lanes) {
+                      const c10::optional<at::Tensor>& w_head, double k_scale, int64_t max_len, int64_t lanes, bool act) {
   const long T = q.size(0);
   TORCH_CHECK(H >= 1 && Hk >= 1 && H % Hk == 0 && dk >= 1 && dk <= 256 && dv >= 1, "delta_scan sizes");
   check_rows(q, T, Hk * dk, "q"); check_rows(k, T, Hk * dk, "k"); check_rows(v, T, H * dv, "v");
@@ -1369,7 +1369,7 @@ at::Tensor delta_scan(const at::Tensor& q, const at::Tensor& k, const at::Tensor
   CHECK_RC(lk_delta_scan(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), esz, wp, ws, pp, ps, zp, zs,
                          wp ? nullptr : fpo(w_head, H, "w_head"), (float)k_scale, state.data_ptr<float>(), ip(cu), ip(slots),
                          ip(positions), cu.numel() - 1, (int)H, (int)Hk, (int)dk, (int)dv, o.data_ptr<float>(), o.stride(0),
-                         wide, cur_stream()), "delta_scan");
+                         wide, act ? 1 : 0, cur_stream()), "delta_scan");
   return o;
 }
 

@@ -36,6 +36,8 @@ LK_DEVICE void stf<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
 template <>
 LK_DEVICE void stf<float>(float* p, float v) { *p = v; }
 
+LK_DEVICE float scan_act(float x, int act) { return act ? x / (1.f + expf(-x)) : x; }
+
 struct ScanParams {
   const void* q;   // rows of Hk * dk
   const void* k;   // rows of Hk * dk
@@ -47,6 +49,7 @@ struct ScanParams {
   long ws, ps, zs;
   const float* w_head;  // [H], used when w is null
   float k_scale;
+  int act;       // 1: q, k and v are silu of what the rows hold (f32, applied as they are staged)
   float* state;  // [slots, H, dk, dv]
   const int* cu;
   const int* slots;
@@ -137,8 +140,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
       const int e = threadIdx.x + 256 * c, t = e / (R * DKT), i = e % (R * DKT);
       const long row = row0 + t0 + t;
       const bool in = i < a.dk && t0 + t < len;
-      pf[c][OQ] = in ? ldf<TQ>(qg + row * a.qs + i) : 0.f;
-      pf[c][OK] = in ? ldf<TQ>(kg + row * a.ks + i) * a.k_scale : 0.f;
+      pf[c][OQ] = in ? scan_act(ldf<TQ>(qg + row * a.qs + i), a.act) : 0.f;
+      pf[c][OK] = in ? scan_act(ldf<TQ>(kg + row * a.ks + i), a.act) * a.k_scale : 0.f;
       if constexpr (FULL) {
         pf[c][OW] = in ? a.w[row * a.ws + (long)h * a.dk + i] : 0.f;
         pf[c][OP] = in ? a.p[row * a.ps + (long)h * a.dk + i] : 0.f;
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
 #pragma unroll
     for (int c = 0; c < CV; ++c) {
       const int e = threadIdx.x + 256 * c, t = e / cols, cc = e % cols;
-      pv[c] = (t < TT && t0 + t < len && j0 + cc < a.dv) ? ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + cc) : 0.f;
+      pv[c] = (t < TT && t0 + t < len && j0 + cc < a.dv) ? scan_act(ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + cc), a.act) : 0.f;
     }
   };
   if constexpr (TILE_PF) gload(0);
@@ -172,8 +175,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
         const int t = e / (R * DKT), i = e % (R * DKT), li = i + 4 * (i / DKT);
         const long row = row0 + t0 + t;
         const bool in = i < a.dk;
-        ops[t][OQ][li] = in ? ldf<TQ>(qg + row * a.qs + i) : 0.f;
-        ops[t][OK][li] = in ? ldf<TQ>(kg + row * a.ks + i) * a.k_scale : 0.f;
+        ops[t][OQ][li] = in ? scan_act(ldf<TQ>(qg + row * a.qs + i), a.act) : 0.f;
+        ops[t][OK][li] = in ? scan_act(ldf<TQ>(kg + row * a.ks + i), a.act) * a.k_scale : 0.f;
         if constexpr (FULL) {
           ops[t][OW][li] = in ? a.w[row * a.ws + (long)h * a.dk + i] : 0.f;
           ops[t][OP][li] = in ? a.p[row * a.ps + (long)h * a.dk + i] : 0.f;
@@ -182,7 +185,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
       }
       for (int e = threadIdx.x; e < nt * cols; e += 256) {
         const int t = e / cols, c = e % cols;
-        vs[t][c] = j0 + c < a.dv ? ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + c) : 0.f;
+        vs[t][c] = j0 + c < a.dv ? scan_act(ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + c), a.act) : 0.f;
       }
     }
     __syncthreads();
@@ -367,6 +370,27 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   }
 }
 
+// The same for fewer heads than waves (one norm over a long row): the whole workgroup takes each head in turn
+template <typename TG, typename TO>
+__global__ __launch_bounds__(256) void row_norm_gate_kernel(const float* __restrict__ o, long os, const TG* __restrict__ g, long gs,
+                                                            const float* __restrict__ w, int H, int dv, float eps, int kind,
+                                                            TO* __restrict__ out, long outs) {
+  __shared__ float red[4];
+  const long t = blockIdx.x;
+  for (int h = 0; h < H; ++h) {
+    const float* x = o + t * os + (long)h * dv;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < dv; c += 256) ss += x[c] * x[c];
+    const float inv = 1.f / sqrtf(block_sum<4>(ss, red) / (float)dv + eps);
+    for (int c = threadIdx.x; c < dv; c += 256) {
+      const long hc = (long)h * dv + c;
+      const float gv = ldf<TG>(g + t * gs + hc);
+      const float s = sigmoid_f(gv);
+      stf<TO>(out + t * outs + hc, x[c] * inv * (w ? w[hc] : 1.f) * (kind == 0 ? gv * s : s));
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void tanh_kernel(T* __restrict__ x, long xs, int n) {
   const long t = blockIdx.x;
@@ -378,14 +402,14 @@ __global__ __launch_bounds__(256) void tanh_kernel(T* __restrict__ x, long xs, i
 int lk_delta_scan(const void* q, long qs, const void* k, long ks, const void* v, long vs, int qkv_esz, const float* w, long ws,
                   const float* p, long ps, const float* z, long zs, const float* w_head, float k_scale, float* state,
                   const int* cu, const int* slots, const int* positions, int S, int H, int Hk, int dk, int dv, float* o, long os,
-                  int wide, hipStream_t st) {
+                  int wide, int act, hipStream_t st) {
   if (S <= 0) return 0;
   if (H < 1 || Hk < 1 || H % Hk || dk < 1 || dk > 256 || dv < 1 || H > 65535) return -1;
   const bool full = w != nullptr;
   if (full ? (p == nullptr || z == nullptr) : (w_head == nullptr || p != nullptr || z != nullptr)) return -1;
   ScanParams a;
   a.q = q; a.k = k; a.v = v; a.qs = qs; a.ks = ks; a.vs = vs;
-  a.w = w; a.p = p; a.z = z; a.ws = ws; a.ps = ps; a.zs = zs; a.w_head = w_head; a.k_scale = k_scale;
+  a.w = w; a.p = p; a.z = z; a.ws = ws; a.ps = ps; a.zs = zs; a.w_head = w_head; a.k_scale = k_scale; a.act = act;
   a.state = state; a.cu = cu; a.slots = slots; a.positions = positions; a.o = o; a.os = os;
   a.H = H; a.Hk = Hk; a.dk = dk; a.dv = dv;
   return qkv_esz == 2 ? scan_t<bf16_t>(a, S, full, wide, st) : scan_t<float>(a, S, full, wide, st);
@@ -425,8 +449,11 @@ int lk_head_norm_gate(const float* o, long os, const void* g, long gs, int g_esz
                       int kind, void* out, long outs, int out_esz, hipStream_t st) {
   if (T <= 0) return 0;
   if (kind != 0 && kind != 1) return -1;
-#define LK_HNG(TG, TO) \
-  head_norm_gate_kernel<TG, TO><<<(unsigned)T, 256, 0, st>>>(o, os, (const TG*)g, gs, w, H, dv, eps, kind, (TO*)out, outs)
+#define LK_HNG(TG, TO)                                                                                                          \
+  if (H < 4 && dv >= 256)                                                                                                       \
+    row_norm_gate_kernel<TG, TO><<<(unsigned)T, 256, 0, st>>>(o, os, (const TG*)g, gs, w, H, dv, eps, kind, (TO*)out, outs);   \
+  else                                                                                                                          \
+    head_norm_gate_kernel<TG, TO><<<(unsigned)T, 256, 0, st>>>(o, os, (const TG*)g, gs, w, H, dv, eps, kind, (TO*)out, outs)
   if (g_esz == 2 && out_esz == 2) LK_HNG(bf16_t, bf16_t);
   else if (g_esz == 4 && out_esz == 4) LK_HNG(float, float);
   else if (g_esz == 2) LK_HNG(bf16_t, float);

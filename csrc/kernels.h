@@ -276,7 +276,7 @@ int lk_dual_rmsnorm_mean(const void* a, long as, const float* wa, const void* b,
 int lk_delta_scan(const void* q, long qs, const void* k, long ks, const void* v, long vs, int qkv_esz, const float* w, long ws,
                   const float* p, long ps, const float* z, long zs, const float* w_head, float k_scale, float* state,
                   const int* cu, const int* slots, const int* positions, int S, int H, int Hk, int dk, int dv, float* o, long os,
-                  int wide, hipStream_t st);
+                  int wide, int act, hipStream_t st);
 int lk_gated_delta_prep(const void* q, long qs, const void* k, long ks, const void* v, long vs, const void* beta, long bs,
                         const void* dt, long dts, const float* dt_bias, const float* A_log, long T, int H, int Hk, int dk, int dv,
                         float* qn, float* kn, float* vb, float* g, float* p, float* z, int esz, hipStream_t st);

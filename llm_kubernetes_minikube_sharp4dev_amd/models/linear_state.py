@@ -114,13 +114,13 @@ class LightningSpec:
 
 
 def lightning_mixer(h, w_in, rows: FusedRows, decay, norm_w, w_out, spec: LightningSpec, eps: float, state, meta, out_dtype):
-    """h [T, W] -> [T, W]: q | k | v | g in one projection, silu on the q | k | v columns in place, the decayed
-    scan (f32 state), one RMS norm over all heads times a weight times sigmoid(g), output projection."""
+    """h [T, W] -> [T, W]: q | k | v | g in one projection, the decayed scan on silu(q), silu(k), silu(v) (the
+    activation is applied in f32 as the scan stages its operands; f32 state), one RMS norm over all heads times a
+    weight times sigmoid(g), output projection."""
     u = ops.linear(h, w_in)
-    ops.silu_(u[:, : rows.off["g"]])          # q | k | v and the zero padding between them (silu(0) = 0)
     o = ops.delta_scan(rows.cols(u, "q"), rows.cols(u, "k"), rows.cols(u, "v"), None, None, None, state[0], meta.seq_cu,
                        meta.state_slots, meta.positions, spec.heads, spec.heads, spec.dim, spec.vdim, w_head=decay,
-                       max_len=meta.max_seq_len)
+                       max_len=meta.max_seq_len, act=True)
     g = ops.head_norm_gate(o, rows.cols(u, "g"), norm_w, 1, eps, ops.GATE_SIGMOID, out_dtype)
     return ops.linear(g, w_out)
 

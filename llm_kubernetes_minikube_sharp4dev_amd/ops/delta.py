@@ -37,16 +37,17 @@ def delta_scan_supported(dk: int, dv: int) -> bool:
 
 
 def delta_scan(q, k, v, w, p, z, state, cu, slots, positions, H: int, Hk: int, dk: int, dv: int,
-               w_head=None, k_scale: float = 1.0, max_len: int = 1, lanes: int = 0):
+               w_head=None, k_scale: float = 1.0, max_len: int = 1, lanes: int = 0, act: bool = False):
     """o f32 [T, H * dv] of the recurrence in the module docstring, per sequence and head, the state read
     from / left in ``state[slot]``.  q, k: rows of ``Hk * dk`` (head h reads q/k head ``h // (H / Hk)``),
     v: rows of ``H * dv``; each in bf16 or f32 (k is multiplied by ``k_scale`` in f32).  ``w``: f32 rows of
     ``H * dk``, or None with ``w_head`` f32 [H] (one decay per head).  ``p``, ``z``: f32 rows of ``H * dk``,
     or both None (no removal term).  ``lanes``: 4 or 16 forces how many lanes of the GPU kernel share a state
-    column (default: by the step's shape -- 16 while (sequence, head) pairs do not fill the chip)."""
+    column (default: by the step's shape -- 16 while (sequence, head) pairs do not fill the chip).  ``act``: q, k
+    and v are the silu (f32) of what the rows hold."""
     if use_hip(q):
         return lib().delta_scan(q, k, v, w, p, z, state, cu, slots, positions, H, Hk, dk, dv, w_head, float(k_scale), int(max_len),
-                                int(lanes))
+                                int(lanes), bool(act))
     T = q.shape[0]
     o = torch.zeros(T, H * dv, dtype=torch.float32, device=q.device)
     cul, sl = cu.tolist(), slots.tolist()
@@ -56,9 +57,10 @@ def delta_scan(q, k, v, w, p, z, state, cu, slots, positions, H: int, Hk: int, d
         if sl[s] < 0 or r1 <= r0:
             continue
         S = state[sl[s]].clone() if int(positions[r0]) > 0 else torch.zeros_like(state[sl[s]])     # [H, dk, dv]
-        qq = q[r0:r1, : Hk * dk].float().view(-1, Hk, dk).repeat_interleave(rep, 1)
-        kk = (k[r0:r1, : Hk * dk].float() * k_scale).view(-1, Hk, dk).repeat_interleave(rep, 1)
-        vv = v[r0:r1, : H * dv].float().view(-1, H, dv)
+        f = F.silu if act else (lambda t: t)
+        qq = f(q[r0:r1, : Hk * dk].float()).view(-1, Hk, dk).repeat_interleave(rep, 1)
+        kk = (f(k[r0:r1, : Hk * dk].float()) * k_scale).view(-1, Hk, dk).repeat_interleave(rep, 1)
+        vv = f(v[r0:r1, : H * dv].float()).view(-1, H, dv)
         ww = w[r0:r1, : H * dk].view(-1, H, dk) if w is not None else w_head.view(1, H, 1).expand(r1 - r0, H, dk)
         for t in range(r1 - r0):
             new = ww[t].unsqueeze(-1) * S + kk[t].unsqueeze(-1) * vv[t].unsqueeze(1)
