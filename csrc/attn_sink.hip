@@ -518,8 +518,10 @@ bool shape_ok(const SinkParams& p, int esz) {
 template <typename T, int PAD>
 int launch_prefill(const SinkParams& p, const int* cu_q, const int* ctx, const int* ts, const int* tq, int ntiles, void* out,
                    long os, hipStream_t st) {
-  // a query that sees at most 512 keys (17 steps): one wave per tile
-  const bool wt = p.mkind != 0 && p.msize <= 512;
+  // a query that sees at most 512 keys (17 steps): one wave per tile.  Likewise when the step has (tile, head) pairs enough to
+  // fill every SIMD of the chip several times with one wave each: splitting a tile's keys over a workgroup then only adds
+  // the merge and leaves each wave a short chain of steps to hide its loads behind
+  const bool wt = (p.mkind != 0 && p.msize <= 512) || (long)ntiles * p.H >= 8192;
   const int gy = wt ? (ntiles + 3) / 4 : ntiles;
   if (gy > 65535) return -2;
   if (wt) sinkattn_prefill_kernel<T, PAD, true><<<dim3(p.H, gy), 256, 0, st>>>(p, cu_q, ctx, ts, tq, ntiles, reinterpret_cast<T*>(out), os);

@@ -36,7 +36,13 @@ LK_DEVICE void stf<bf16_t>(bf16_t* p, float v) { *p = f2bf(v); }
 template <>
 LK_DEVICE void stf<float>(float* p, float v) { *p = v; }
 
-LK_DEVICE float scan_act(float x, int act) { return act ? x / (1.f + expf(-x)) : x; }
+// silu of a staged operand: accurate exponential for f32 rows, the hardware one for bf16 rows (whose own rounding is 2^-9)
+template <typename TQ>
+LK_DEVICE float scan_act(float x, int act) {
+  if (!act) return x;
+  if constexpr (sizeof(TQ) == 4) return x / (1.f + expf(-x));
+  else return x * __builtin_amdgcn_rcpf(1.f + __expf(-x));
+}
 
 struct ScanParams {
   const void* q;   // rows of Hk * dk
@@ -140,8 +146,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
       const int e = threadIdx.x + 256 * c, t = e / (R * DKT), i = e % (R * DKT);
       const long row = row0 + t0 + t;
       const bool in = i < a.dk && t0 + t < len;
-      pf[c][OQ] = in ? scan_act(ldf<TQ>(qg + row * a.qs + i), a.act) : 0.f;
-      pf[c][OK] = in ? scan_act(ldf<TQ>(kg + row * a.ks + i), a.act) * a.k_scale : 0.f;
+      pf[c][OQ] = in ? scan_act<TQ>(ldf<TQ>(qg + row * a.qs + i), a.act) : 0.f;
+      pf[c][OK] = in ? scan_act<TQ>(ldf<TQ>(kg + row * a.ks + i), a.act) * a.k_scale : 0.f;
       if constexpr (FULL) {
         pf[c][OW] = in ? a.w[row * a.ws + (long)h * a.dk + i] : 0.f;
         pf[c][OP] = in ? a.p[row * a.ps + (long)h * a.dk + i] : 0.f;
@@ -151,7 +157,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
 #pragma unroll
     for (int c = 0; c < CV; ++c) {
       const int e = threadIdx.x + 256 * c, t = e / cols, cc = e % cols;
-      pv[c] = (t < TT && t0 + t < len && j0 + cc < a.dv) ? scan_act(ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + cc), a.act) : 0.f;
+      pv[c] = (t < TT && t0 + t < len && j0 + cc < a.dv) ? scan_act<TQ>(ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + cc), a.act) : 0.f;
     }
   };
   if constexpr (TILE_PF) gload(0);
@@ -175,8 +181,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
         const int t = e / (R * DKT), i = e % (R * DKT), li = i + 4 * (i / DKT);
         const long row = row0 + t0 + t;
         const bool in = i < a.dk;
-        ops[t][OQ][li] = in ? scan_act(ldf<TQ>(qg + row * a.qs + i), a.act) : 0.f;
-        ops[t][OK][li] = in ? scan_act(ldf<TQ>(kg + row * a.ks + i), a.act) * a.k_scale : 0.f;
+        ops[t][OQ][li] = in ? scan_act<TQ>(ldf<TQ>(qg + row * a.qs + i), a.act) : 0.f;
+        ops[t][OK][li] = in ? scan_act<TQ>(ldf<TQ>(kg + row * a.ks + i), a.act) * a.k_scale : 0.f;
         if constexpr (FULL) {
           ops[t][OW][li] = in ? a.w[row * a.ws + (long)h * a.dk + i] : 0.f;
           ops[t][OP][li] = in ? a.p[row * a.ps + (long)h * a.dk + i] : 0.f;
@@ -185,7 +191,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(ScanParams a) {
       }
       for (int e = threadIdx.x; e < nt * cols; e += 256) {
         const int t = e / cols, c = e % cols;
-        vs[t][c] = j0 + c < a.dv ? scan_act(ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + c), a.act) : 0.f;
+        vs[t][c] = j0 + c < a.dv ? scan_act<TQ>(ldf<TQ>(vg + (long)(row0 + t0 + t) * a.vs + j0 + c), a.act) : 0.f;
       }
     }
     __syncthreads();

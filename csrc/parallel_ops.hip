@@ -177,13 +177,14 @@ template <typename T>
 __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ h, long hs, const float* __restrict__ wr, int E, int W,
                                                           long rows, int top, int groups, int keep, float scale,
                                                           int* __restrict__ experts, float* __restrict__ weights) {
-  extern __shared__ float hrow[];                    // [kRouterTok][W]
+  extern __shared__ __attribute__((aligned(16))) float hrow[];   // [kRouterTok][W]
+  const bool vec = W % 4 == 0 && reinterpret_cast<uintptr_t>(wr) % 16 == 0;
   __shared__ float sc[kRouterTok][kRouterMaxE];      // sigmoid scores
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const long t0 = (long)blockIdx.x * kRouterTok;
-  for (int i = threadIdx.x; i < kRouterTok * W; i += 256) {
-    const long t = t0 + i / W;
-    hrow[i] = t < rows ? ldv<T>(h + t * hs + i % W) : 0.f;
+  for (int k = 0; k < kRouterTok; ++k) {
+    const long t = t0 + k;
+    for (int c = threadIdx.x; c < W; c += 256) hrow[k * W + c] = t < rows ? ldv<T>(h + t * hs + c) : 0.f;
   }
   __syncthreads();
   for (int e = wv; e < E; e += 4) {
@@ -191,10 +192,29 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ 
     float acc[kRouterTok];
 #pragma unroll
     for (int k = 0; k < kRouterTok; ++k) acc[k] = 0.f;
-    for (int c = lane; c < W; c += 64) {
-      const float w = wrow[c];
+    if (vec) {   // 16-byte loads of the weight row, four of them requested before the first is used
+      const int nv = W >> 2;
+      for (int c0 = lane; c0 < nv; c0 += 256) {
+        floatx4 w4[4];
 #pragma unroll
-      for (int k = 0; k < kRouterTok; ++k) acc[k] += w * hrow[k * W + c];
+        for (int u = 0; u < 4; ++u)
+          w4[u] = c0 + 64 * u < nv ? *reinterpret_cast<const floatx4*>(wrow + 4 * (c0 + 64 * u)) : floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = min(c0 + 64 * u, nv - 1);   // rows past the end multiply zeros
+#pragma unroll
+          for (int k = 0; k < kRouterTok; ++k) {
+            const floatx4 hv = *reinterpret_cast<const floatx4*>(hrow + k * W + 4 * c);
+            acc[k] += (w4[u][0] * hv[0] + w4[u][1] * hv[1]) + (w4[u][2] * hv[2] + w4[u][3] * hv[3]);
+          }
+        }
+      }
+    } else {
+      for (int c = lane; c < W; c += 64) {
+        const float w = wrow[c];
+#pragma unroll
+        for (int k = 0; k < kRouterTok; ++k) acc[k] += w * hrow[k * W + c];
+      }
     }
 #pragma unroll
     for (int k = 0; k < kRouterTok; ++k) {
