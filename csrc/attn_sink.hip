@@ -65,13 +65,6 @@ struct SinkParams {
 
 LK_DEVICE int blocks_seen(int qpos, int msize, int pool) { return max(0, qpos - msize + 1) / pool; }
 
-LK_DEVICE SinkParams pooled_view(const SinkParams& p) {
-  SinkParams r = p;
-  r.kc = p.pkc;
-  r.vc = p.pvc;
-  return r;
-}
-
 LK_DEVICE int first_key(int qpos, int mkind, int msize) {
   if (mkind == 1) return (qpos / msize) * msize;
   if (mkind == 2) return max(0, qpos - msize + 1);
@@ -97,14 +90,14 @@ LK_DEVICE float cap_f(float s, float cap, float icap) {
 // the O^T accumulators.  Key order inside a step: see attn_sigmoid.hip (lane group g holds the weights
 // of the 8 consecutive keys 8g .. 8g + 7).
 template <typename T, int PAD>
-LK_DEVICE void sink_run(const SinkParams& p, const uint4_t (&qf)[PAD / (4 * El<T>::V)], int kvh, const int* bt, int k0, int k1,
-                        int step0, int stride, bool cvalid, int qpos, int klo, float hs, float& m, float& l,
-                        floatx4 (&o)[PAD / 16]) {
+LK_DEVICE void sink_run(const SinkParams& p, const void* kcache, const void* vcache, const uint4_t (&qf)[PAD / (4 * El<T>::V)], int kvh,
+                        const int* bt, int k0, int k1, int step0, int stride, bool cvalid, int qpos, int klo, float hs, float& m,
+                        float& l, floatx4 (&o)[PAD / 16]) {
   constexpr int EV = El<T>::V, KS = PAD / (4 * EV), VT = PAD / 16;
   constexpr bool BF = sizeof(T) == 2;
   const int lane = threadIdx.x & 63, n16 = lane & 15, g = lane >> 4;
-  const T* kc = reinterpret_cast<const T*>(p.kc);
-  const T* vc = reinterpret_cast<const T*>(p.vc);
+  const T* kc = reinterpret_cast<const T*>(kcache);
+  const T* vc = reinterpret_cast<const T*>(vcache);
   const int krow = 8 * (n16 >> 2) + (n16 & 3);
   // bf16: the next step's K fragments are requested as soon as this step's Q.K products have consumed the
   // current ones, and this step's V fragments before the softmax arithmetic, so both fly under it
@@ -301,20 +294,19 @@ __global__ __launch_bounds__(256) void sinkattn_prefill_kernel(SinkParams p, con
   float m = p.sink ? 0.f : kNegBig, l = 0.f;
   const int k1 = min(ctx, past + q0 + 16);
   const int k0 = first_key(past + q0, p.mkind, p.msize) & ~31;   // first(i) never decreases with i
-  sink_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, k0, k1, WT ? 0 : w, WT ? 1 : 4, cvalid, qpos,
-                   first_key(qpos, p.mkind, p.msize), p.hscale[head], m, l, o);
-  if (p.pool > 0) {
-    const int nbt = blocks_seen(k1 - 1, p.msize, p.pool);   // the tile's last query sees the most blocks
-    if (nbt > 0)
-      sink_run<T, PAD>(pooled_view(p), qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, nbt, WT ? 0 : w, WT ? 1 : 4,
-                       cvalid, blocks_seen(qpos, p.msize, p.pool) - 1, 0, p.hscale[head], m, l, o);
-  }
+  const int klo_q = first_key(qpos, p.mkind, p.msize);
+  sink_run<T, PAD>(p, p.kc, p.vc, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, k0, k1, WT ? 0 : w, WT ? 1 : 4, cvalid, qpos, klo_q,
+                   p.hscale[head], m, l, o);
   {
-    // kept first positions behind the window: the tile's last query has the latest window, so it bounds the pass
-    const int nk = kept_keys(p, first_key(k1 - 1, p.mkind, p.msize));
-    if (nk > 0)
-      sink_run<T, PAD>(p, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, nk, WT ? 0 : w, WT ? 1 : 4, cvalid,
-                       kept_keys(p, first_key(qpos, p.mkind, p.msize)) - 1, 0, p.hscale[head], m, l, o);
+    // A second pass over what lies behind the window -- the pooled blocks it has left behind entirely, or (never both) the kept
+    // first positions: entries [0, n1) of the pooled / the plain cache pair, bounded by the tile's last query (it sees the most
+    // blocks and has the latest window) and per column by its own window.
+    const bool pooled = p.pool > 0;
+    const int n1 = pooled ? blocks_seen(k1 - 1, p.msize, p.pool) : kept_keys(p, first_key(k1 - 1, p.mkind, p.msize));
+    const int vis = (pooled ? blocks_seen(qpos, p.msize, p.pool) : kept_keys(p, klo_q)) - 1;
+    if (n1 > 0)
+      sink_run<T, PAD>(p, pooled ? p.pkc : p.kc, pooled ? p.pvc : p.vc, qf, head / (p.H / p.G), p.bt + (long)b * p.bt_stride, 0, n1,
+                       WT ? 0 : w, WT ? 1 : 4, cvalid, vis, 0, p.hscale[head], m, l, o);
   }
   if constexpr (WT) {
     l += __shfl_xor(l, 16, 64);
@@ -360,21 +352,18 @@ __global__ __launch_bounds__(256) void sinkattn_decode_kernel(SinkParams p, cons
   for (int vt = 0; vt < VT; ++vt) o[vt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m = p.sink ? 0.f : kNegBig, l = 0.f;
   const int klo = first_key(ctx - 1, p.mkind, p.msize), k0 = klo & ~31;
-  // the key splits share the window's 32-key steps and, behind them, the steps over the pooled blocks
-  // and, behind those, the steps over the kept first positions that the window has left
-  const int nb = p.pool > 0 ? blocks_seen(ctx - 1, p.msize, p.pool) : 0;
-  const int nk = kept_keys(p, klo);
-  const int nwin = (ctx - k0 + 31) / 32, e1 = nwin + (nb + 31) / 32, nsteps = e1 + (nk + 31) / 32, spz = (nsteps + Z - 1) / Z;
+  // the key splits share the window's 32-key steps and, behind them, the steps over what lies behind the window: the pooled
+  // blocks or (never both) the kept first positions, entries [0, n1) of the pooled / the plain cache pair
+  const bool pooled = p.pool > 0;
+  const int n1 = pooled ? blocks_seen(ctx - 1, p.msize, p.pool) : kept_keys(p, klo);
+  const int nwin = (ctx - k0 + 31) / 32, nsteps = nwin + (n1 + 31) / 32, spz = (nsteps + Z - 1) / Z;
   const int s0 = z * spz, s1 = min(nsteps, s0 + spz);
   if (s0 < min(s1, nwin))
-    sink_run<T, PAD>(p, qf, kvh, p.bt + (long)b * p.bt_stride, k0 + 32 * s0, min(ctx, k0 + 32 * min(s1, nwin)), w, 4, cvalid, ctx - 1,
-                     klo, p.hscale[head], m, l, o);
-  if (max(s0, nwin) < min(s1, e1))
-    sink_run<T, PAD>(pooled_view(p), qf, kvh, p.bt + (long)b * p.bt_stride, 32 * (max(s0, nwin) - nwin), min(nb, 32 * (min(s1, e1) - nwin)),
-                     w, 4, cvalid, nb - 1, 0, p.hscale[head], m, l, o);
-  if (max(s0, e1) < s1)
-    sink_run<T, PAD>(p, qf, kvh, p.bt + (long)b * p.bt_stride, 32 * (max(s0, e1) - e1), min(nk, 32 * (s1 - e1)), w, 4, cvalid, nk - 1, 0,
-                     p.hscale[head], m, l, o);
+    sink_run<T, PAD>(p, p.kc, p.vc, qf, kvh, p.bt + (long)b * p.bt_stride, k0 + 32 * s0, min(ctx, k0 + 32 * min(s1, nwin)), w, 4, cvalid,
+                     ctx - 1, klo, p.hscale[head], m, l, o);
+  if (max(s0, nwin) < s1)
+    sink_run<T, PAD>(p, pooled ? p.pkc : p.kc, pooled ? p.pvc : p.vc, qf, kvh, p.bt + (long)b * p.bt_stride, 32 * (max(s0, nwin) - nwin),
+                     min(n1, 32 * (s1 - nwin)), w, 4, cvalid, n1 - 1, 0, p.hscale[head], m, l, o);
   merge_waves<EXACT, VT>(m, l, o, red, ml);
   if (w == 0 && cvalid) {
     if (Z == 1) {
@@ -521,7 +510,7 @@ int launch_prefill(const SinkParams& p, const int* cu_q, const int* ctx, const i
   // a query that sees at most 512 keys (17 steps): one wave per tile.  Likewise when the step has (tile, head) pairs enough to
   // fill every SIMD of the chip several times with one wave each: splitting a tile's keys over a workgroup then only adds
   // the merge and leaves each wave a short chain of steps to hide its loads behind
-  const bool wt = (p.mkind != 0 && p.msize <= 512) || (long)ntiles * p.H >= 8192;
+  const bool wt = (p.mkind != 0 && p.msize <= 512) || (long)ntiles * p.H >= 2048;
   const int gy = wt ? (ntiles + 3) / 4 : ntiles;
   if (gy > 65535) return -2;
   if (wt) sinkattn_prefill_kernel<T, PAD, true><<<dim3(p.H, gy), 256, 0, st>>>(p, cu_q, ctx, ts, tq, ntiles, reinterpret_cast<T*>(out), os);
