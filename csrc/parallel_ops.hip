@@ -171,15 +171,15 @@ LK_DEVICE void wave_argmax(float& s, int& i) {
   }
 }
 
-// grid = ceil(T / kRouterTok); dynamic LDS: kRouterTok rows of W floats.  The 4 waves take the experts in turn
-// (lanes stride the width, 4 accumulators per expert), then wave w makes the choice of token w.
+// grid = ceil(T / kRouterTok); dynamic LDS: kRouterTok rows of W floats and of E scores.  The 4 waves take the experts in
+// blocks of 4 (lanes stride the width), then wave w makes the choice of token w.
 template <typename T>
 __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ h, long hs, const float* __restrict__ wr, int E, int W,
                                                           long rows, int top, int groups, int keep, float scale,
                                                           int* __restrict__ experts, float* __restrict__ weights) {
-  extern __shared__ __attribute__((aligned(16))) float hrow[];   // [kRouterTok][W]
+  extern __shared__ __attribute__((aligned(16))) float hrow[];   // [kRouterTok][W], then the sigmoid scores [kRouterTok][E]
+  float* sc = hrow + (long)kRouterTok * W;
   const bool vec = W % 4 == 0 && reinterpret_cast<uintptr_t>(wr) % 16 == 0;
-  __shared__ float sc[kRouterTok][kRouterMaxE];      // sigmoid scores
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const long t0 = (long)blockIdx.x * kRouterTok;
   for (int k = 0; k < kRouterTok; ++k) {
@@ -187,45 +187,59 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ 
     for (int c = threadIdx.x; c < W; c += 256) hrow[k * W + c] = t < rows ? ldv<T>(h + t * hs + c) : 0.f;
   }
   __syncthreads();
-  for (int e = wv; e < E; e += 4) {
-    const float* wrow = wr + (long)e * W;
-    float acc[kRouterTok];
+  // a wave takes blocks of 4 experts; per round of the width the 16 weight loads (4 experts x 4 x 16 bytes per lane) are
+  // requested together and a row fragment read from LDS serves the 4 experts
+  for (int eb = wv * 4; eb < E; eb += 16) {
+    float acc[4][kRouterTok];
 #pragma unroll
-    for (int k = 0; k < kRouterTok; ++k) acc[k] = 0.f;
-    if (vec) {   // 16-byte loads of the weight row, four of them requested before the first is used
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+      for (int k = 0; k < kRouterTok; ++k) acc[x][k] = 0.f;
+    if (vec) {
       const int nv = W >> 2;
       for (int c0 = lane; c0 < nv; c0 += 256) {
-        floatx4 w4[4];
+        floatx4 w4[4][4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-          w4[u] = c0 + 64 * u < nv ? *reinterpret_cast<const floatx4*>(wrow + 4 * (c0 + 64 * u)) : floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int x = 0; x < 4; ++x) {
+          const float* wrow = wr + (long)min(eb + x, E - 1) * W;
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            w4[x][u] = c0 + 64 * u < nv ? *reinterpret_cast<const floatx4*>(wrow + 4 * (c0 + 64 * u)) : floatx4{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          const int c = min(c0 + 64 * u, nv - 1);   // rows past the end multiply zeros
+          const int c = min(c0 + 64 * u, nv - 1);   // columns past the end multiply zero weights
 #pragma unroll
           for (int k = 0; k < kRouterTok; ++k) {
             const floatx4 hv = *reinterpret_cast<const floatx4*>(hrow + k * W + 4 * c);
-            acc[k] += (w4[u][0] * hv[0] + w4[u][1] * hv[1]) + (w4[u][2] * hv[2] + w4[u][3] * hv[3]);
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+              acc[x][k] += (w4[x][u][0] * hv[0] + w4[x][u][1] * hv[1]) + (w4[x][u][2] * hv[2] + w4[x][u][3] * hv[3]);
           }
         }
       }
     } else {
       for (int c = lane; c < W; c += 64) {
-        const float w = wrow[c];
 #pragma unroll
-        for (int k = 0; k < kRouterTok; ++k) acc[k] += w * hrow[k * W + c];
+        for (int x = 0; x < 4; ++x) {
+          const float w = wr[(long)min(eb + x, E - 1) * W + c];
+#pragma unroll
+          for (int k = 0; k < kRouterTok; ++k) acc[x][k] += w * hrow[k * W + c];
+        }
       }
     }
 #pragma unroll
-    for (int k = 0; k < kRouterTok; ++k) {
-      const float z = wave_sum(acc[k]);
-      if (lane == 0) sc[k][e] = 1.f / (1.f + expf(-z));
-    }
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+      for (int k = 0; k < kRouterTok; ++k) {
+        const float z = wave_sum(acc[x][k]);
+        if (lane == 0 && eb + x < E) sc[k * E + eb + x] = 1.f / (1.f + expf(-z));
+      }
   }
   __syncthreads();
   const long t = t0 + wv;
   if (t >= rows) return;
-  float* s = sc[wv];
+  float* s = sc + (long)wv * E;
   const int per = E / groups;
   if (groups > 1) {
     // lane g: the sum of group g's two largest scores (at most 64 groups, checked on the host)
@@ -330,7 +344,7 @@ int lk_router_topk(const void* h, long hs, const float* wr, int E, int W, long r
   if (E < 1 || E > kRouterMaxE || W < 1 || groups < 1 || groups > 64 || E % groups || keep < 1 || keep > groups || top < 1 ||
       top > kRouterMaxTop || top > (E / groups) * keep)
     return -1;
-  const size_t lds = (size_t)kRouterTok * W * sizeof(float);
+  const size_t lds = (size_t)kRouterTok * (W + E) * sizeof(float);
   if (lds > 128 * 1024) return -1;
   const unsigned grid = (unsigned)((rows + kRouterTok - 1) / kRouterTok);
   if (esz == 2) {
