@@ -187,7 +187,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ 
     for (int c = threadIdx.x; c < W; c += 256) hrow[k * W + c] = t < rows ? ldv<T>(h + t * hs + c) : 0.f;
   }
   __syncthreads();
-  // a wave takes blocks of 4 experts; per round of the width the 16 weight loads (4 experts x 4 x 16 bytes per lane) are
+  // a wave takes blocks of 4 experts; per pass over the width the 16 weight loads (4 experts x 4 x 16 bytes per lane) are
   // requested together and a row fragment read from LDS serves the 4 experts
   for (int eb = wv * 4; eb < E; eb += 16) {
     float acc[4][kRouterTok];

@@ -64,8 +64,8 @@ CONFIGS = {
     # layers that blend values (the second blends the first's in); dense and routed feed-forwards, groups of 2 of which 2 of 3
     # are kept, a shared expert
     "tri": config([dense(att(4, 2, 24, 16, 0.25, 20, 3, 8.0, True), 40, 1.2),
-                   moe(lat(3, 12, 8, 20, 24, 20, 0.3, 40.0), 20, 6, 2, 3, 2, 1.5, 24),
-                   moe(lig(3, 8, 12, [0.7, 0.93, 0.995]), 20, 6, 2, 3, 2, 1.5, 24),
+                   moe(lat(3, 12, 8, 20, 24, 20, 0.3, 40.0), 20, 6, 2, 3, 2, 1.3, 24),
+                   moe(lig(3, 8, 12, [0.7, 0.93, 0.995]), 20, 6, 2, 3, 2, 1.3, 24),
                    moe(att(4, 2, 24, 16, 0.25, 20, 3, 8.0, True), 20, 6, 3, 2, 2, 0.8)], 48),
     # the lightning mixer first and without a feed-forward; one head everywhere; one expert of one; a window of 7 that keeps
     # nothing, no cap, no blending; then a layer that would blend but is the only one (keeps its own), keep_first = window;
@@ -82,10 +82,10 @@ CONFIGS = {
                     moe(att(2, 1, 72, 40, 0.15, 4096, 2, 0.0, True), 24, 3, 1, shared=16),
                     dense(att(2, 2, 40, 72, 0.15, 9, 14), 24, 2.0)], 56, vocab=130),
     # projections the MFMA / weight-streaming kernels tile: no vendor GEMM, decode steps captured in hipGraphs
-    "mid": config([moe(att(4, 2, 64, 64, 0.125, 48, 4, 20.0, True), 128, 8, 2, 4, 2, 1.5, 128),
-                   moe(lat(4, 64, 32, 64, 256, 256, 0.1, 10000.0), 128, 8, 2, 4, 2, 1.5, 128),
-                   moe(lig(4, 64, 64, [0.9, 0.95, 0.99, 0.999]), 128, 8, 2, 4, 2, 1.5, 128),
-                   dense(att(4, 2, 64, 64, 0.125, 48, 4, 20.0, True), 256, 4.0)], 256, vocab=768),
+    "mid": config([moe(att(4, 2, 64, 64, 0.11, 48, 4, 25.0, True), 128, 8, 2, 4, 2, 1.25, 256),
+                   moe(lat(4, 64, 32, 64, 256, 256, 0.1, 10000.0), 128, 8, 2, 4, 2, 1.25, 256),
+                   moe(lig(4, 64, 64, [0.9, 0.95, 0.99, 0.9985]), 128, 8, 2, 4, 2, 1.25, 256),
+                   dense(att(4, 2, 64, 64, 0.11, 48, 4, 25.0, True), 256, 4.0)], 256, vocab=768),
 }
 _models = {}
 

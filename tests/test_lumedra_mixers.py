@@ -184,7 +184,7 @@ def test_value_blend_in_the_cache_write(device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", ALL)
-@pytest.mark.parametrize("E,groups,keep,top", [(16, 4, 3, 2), (6, 3, 2, 2), (4, 4, 2, 2), (8, 1, 1, 3), (5, 1, 1, 5), (64, 8, 4, 8), (1, 1, 1, 1),
+@pytest.mark.parametrize("E,groups,keep,top", [(16, 4, 2, 3), (6, 3, 2, 2), (4, 4, 2, 2), (8, 1, 1, 3), (5, 1, 1, 5), (64, 8, 4, 8), (1, 1, 1, 1),
                                               (12, 2, 1, 6)])
 def test_router_against_the_oracle(E, groups, keep, top, device, dtype):
     g = torch.Generator().manual_seed(E)
@@ -248,10 +248,10 @@ def test_stream_update_with_both_norms(W, top, device, dtype):
 def test_clamped_gated_activation_and_elementwise_ops(device, dtype):
     g = torch.Generator().manual_seed(4)
     gu = q16(rnd(g, 7, 2 * 52, scale=3.0))
-    got = ops.clamped_glu(gu.to(dtype).to(device), 1.5, 1.702)
-    gg, uu = gu[:, :52].clamp(max=1.5), gu[:, 52:].clamp(-1.5, 1.5)
+    got = ops.clamped_glu(gu.to(dtype).to(device), 1.3, 1.702)
+    gg, uu = gu[:, :52].clamp(max=1.3), gu[:, 52:].clamp(-1.3, 1.3)
     assert rel_err(got, gg * O.sigmoid(1.702 * gg) * (uu + 1)) < tol(dtype)
-    assert float(got.float().max()) <= 1.5 * 2.5 + 0.05            # both clamps bound the result
+    assert float(got.float().max()) <= 1.3 * 2.3 + 0.05            # both clamps bound the result
     x = q16(rnd(g, 5, 40))
     buf = x.to(dtype).to(device).clone()
     ops.silu_(buf[:, 8:32])
