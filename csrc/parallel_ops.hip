@@ -2,7 +2,7 @@
 // the stores is f32):
 //
 //   lk_stream_parallel_norm  x += a + b + sum_k yw[t, k] y[t top + k];  o1 = rms(x) w1,  o2 = rms(x) w2   (one root)
-//   lk_router_topk           z = W_router h (f32), s = sigmoid(z); experts in equal groups of neighbours, a group's
+//   lk_router_topk           z = W_router h (f32), s = sigmoid(z) (evaluated in f64); experts in equal groups of neighbours, a group's
 //                            score = the sum of its two largest s, only the `keep` best groups can be chosen; the
 //                            `top` largest s among those; weights s / (sum of the chosen s + 1e-20) * scale
 //   lk_clamped_glu           g = min(gate, limit), u = clamp(up, -limit, limit):  g sigmoid(alpha g) (u + 1)
@@ -159,10 +159,10 @@ constexpr int kRouterMaxE = 1024;
 constexpr int kRouterMaxTop = 64;
 
 // (score, index) -> the lane pair with the larger score, the smaller index on equal scores
-LK_DEVICE void wave_argmax(float& s, int& i) {
+LK_DEVICE void wave_argmax(double& s, int& i) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
-    const float so = __shfl_xor(s, o, 64);
+    const double so = __shfl_xor(s, o, 64);
     const int io = __shfl_xor(i, o, 64);
     if (so > s || (so == s && io < i)) {
       s = so;
@@ -177,8 +177,12 @@ template <typename T>
 __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ h, long hs, const float* __restrict__ wr, int E, int W,
                                                           long rows, int top, int groups, int keep, float scale,
                                                           int* __restrict__ experts, float* __restrict__ weights) {
-  extern __shared__ __attribute__((aligned(16))) float hrow[];   // [kRouterTok][W], then the sigmoid scores [kRouterTok][E]
-  float* sc = hrow + (long)kRouterTok * W;
+  // [kRouterTok][W] rows, then the f32 logits [kRouterTok][E], then the scores [kRouterTok][E].  The logits are f32 sums of f32
+  // products; the sigmoid, the group sums and the weights are evaluated in f64: an f32 sigmoid near 1 keeps 6e-8 of absolute
+  // resolution where neighbouring scores differ by less, so it would tie logits that are clearly apart
+  extern __shared__ __attribute__((aligned(16))) float hrow[];
+  float* zs = hrow + (long)kRouterTok * W;
+  double* sc = reinterpret_cast<double*>(zs + (long)kRouterTok * E);
   const bool vec = W % 4 == 0 && reinterpret_cast<uintptr_t>(wr) % 16 == 0;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const long t0 = (long)blockIdx.x * kRouterTok;
@@ -233,29 +237,31 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ 
 #pragma unroll
       for (int k = 0; k < kRouterTok; ++k) {
         const float z = wave_sum(acc[x][k]);
-        if (lane == 0 && eb + x < E) sc[k * E + eb + x] = 1.f / (1.f + expf(-z));
+        if (lane == 0 && eb + x < E) zs[k * E + eb + x] = z;
       }
   }
   __syncthreads();
+  for (int i = threadIdx.x; i < kRouterTok * E; i += 256) sc[i] = 1.0 / (1.0 + exp(-(double)zs[i]));
+  __syncthreads();
   const long t = t0 + wv;
   if (t >= rows) return;
-  float* s = sc + (long)wv * E;
+  double* s = sc + (long)wv * E;
   const int per = E / groups;
   if (groups > 1) {
     // lane g: the sum of group g's two largest scores (at most 64 groups, checked on the host)
-    float mine = -3.f;
+    double mine = -3.0;
     if (lane < groups) {
-      float b1 = -1.f, b2 = -1.f;
+      double b1 = -1.0, b2 = -1.0;
       for (int j = 0; j < per; ++j) {
-        const float v = s[lane * per + j];
+        const double v = s[lane * per + j];
         if (v > b1) { b2 = b1; b1 = v; } else if (v > b2) { b2 = v; }
       }
-      mine = b1 + (per > 1 ? b2 : 0.f);
+      mine = b1 + (per > 1 ? b2 : 0.0);
     }
     // pick the `keep` best groups; the others' scores are struck out (-1 < any sigmoid)
     bool kept = false;
     for (int r = 0; r < keep; ++r) {
-      float bs = kept ? -3.f : mine;
+      double bs = kept ? -3.0 : mine;
       int bi = lane;
       wave_argmax(bs, bi);
       if (bi == lane) kept = true;
@@ -263,30 +269,30 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const T* __restrict__ 
     for (int g = 0; g < groups; ++g) {
       const bool kg = __shfl((int)kept, g, 64) != 0;
       if (!kg)
-        for (int j = lane; j < per; j += 64) s[g * per + j] = -1.f - s[g * per + j];   // struck out: below every live score
+        for (int j = lane; j < per; j += 64) s[g * per + j] = -1.0 - s[g * per + j];   // struck out: below every live score
     }
     __builtin_amdgcn_wave_barrier();
   }
   // top experts among the scores left: `top` rounds of a wave-wide argmax
-  float chosen_s = 0.f;   // lane r holds the r-th choice
+  double chosen_s = 0.0;   // lane r holds the r-th choice
   int chosen_e = 0;
-  float sum = 0.f;
+  double sum = 0.0;
   for (int r = 0; r < top; ++r) {
-    float bs = -2.f;
+    double bs = -2.0;
     int bi = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
-      const float v = s[e];
-      if (v >= 0.f && (v > bs || (v == bs && e < bi))) { bs = v; bi = e; }
+      const double v = s[e];
+      if (v >= 0.0 && (v > bs || (v == bs && e < bi))) { bs = v; bi = e; }
     }
     wave_argmax(bs, bi);
     if (bi >= E) bi = 0;                       // nothing left to choose (NaN scores): keep the indices in range
-    else if (lane == (bi & 63)) s[bi] = -1.f - s[bi];
+    else if (lane == (bi & 63)) s[bi] = -1.0 - s[bi];
     if (lane == r) { chosen_s = bs; chosen_e = bi; }
     sum += bs;
   }
   if (lane < top) {
     experts[t * top + lane] = chosen_e;
-    weights[t * top + lane] = chosen_s / (sum + 1e-20f) * scale;
+    weights[t * top + lane] = (float)(chosen_s / (sum + 1e-20) * (double)scale);
   }
 }
 
@@ -344,7 +350,7 @@ int lk_router_topk(const void* h, long hs, const float* wr, int E, int W, long r
   if (E < 1 || E > kRouterMaxE || W < 1 || groups < 1 || groups > 64 || E % groups || keep < 1 || keep > groups || top < 1 ||
       top > kRouterMaxTop || top > (E / groups) * keep)
     return -1;
-  const size_t lds = (size_t)kRouterTok * (W + E) * sizeof(float);
+  const size_t lds = (size_t)kRouterTok * ((W + E) * sizeof(float) + E * sizeof(double));
   if (lds > 128 * 1024) return -1;
   const unsigned grid = (unsigned)((rows + kRouterTok - 1) / kRouterTok);
   if (esz == 2) {

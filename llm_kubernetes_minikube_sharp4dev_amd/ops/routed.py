@@ -48,16 +48,18 @@ def stream_parallel_norm(x, a, b, y, y_w, w1, w2, eps: float, out_dtype=torch.bf
 
 def router_topk(h, w_router, top: int, groups: int = 1, keep: int = 1, scale: float = 1.0):
     """(experts int32 [T, top], weights f32 [T, top]) for rows ``h`` [T, W] and ``w_router`` f32 [E, W]:
-    scores ``s = sigmoid(W_router h)`` in f32; the experts form ``groups`` equal groups of neighbours, a group's
-    score is the sum of its two largest scores and only experts of the ``keep`` best groups can be chosen; the
-    ``top`` largest scores among those; weights ``s / (sum of the chosen s + 1e-20) * scale``."""
+    scores ``s = sigmoid(W_router h)`` from f32 logits (the sigmoid, sums and weights are evaluated in f64); the
+    experts form ``groups`` equal groups of neighbours, a group's score is the sum of its two largest scores and
+    only experts of the ``keep`` best groups can be chosen; the ``top`` largest scores among those; weights
+    ``s / (sum of the chosen s + 1e-20) * scale``."""
     E = w_router.shape[0]
     if E % groups or not 1 <= keep <= groups or not 1 <= top <= (E // groups) * keep:
         raise ValueError(f"router: {top} of {E} experts in {keep} of {groups} groups")
     if use_hip(h):
         ex, wt = lib().router_topk(h, w_router, int(top), int(groups), int(keep), float(scale))
         return ex, wt
-    s = torch.sigmoid(h.float() @ w_router.float().T)                       # [T, E]
+    # f32 logits; the sigmoid and the sums in f64 (an f32 sigmoid near 1 would tie logits that are clearly apart)
+    s = torch.sigmoid((h.float() @ w_router.float().T).double())            # [T, E]
     T = s.shape[0]
     if groups > 1:
         per = E // groups
@@ -69,7 +71,7 @@ def router_topk(h, w_router, top: int, groups: int = 1, keep: int = 1, scale: fl
         sel = s
     ex = sel.topk(top, dim=-1).indices
     sc = s.gather(1, ex)
-    return ex.to(torch.int32), sc / (sc.sum(-1, keepdim=True) + WEIGHT_SUM_FLOOR) * scale
+    return ex.to(torch.int32), (sc / (sc.sum(-1, keepdim=True) + WEIGHT_SUM_FLOOR) * scale).float()
 
 
 def routed_experts(h, experts, w_gate_up, w_down):
