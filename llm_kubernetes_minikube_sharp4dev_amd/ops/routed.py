@@ -64,12 +64,12 @@ def router_topk(h, w_router, top: int, groups: int = 1, keep: int = 1, scale: fl
     if groups > 1:
         per = E // groups
         gs = s.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
-        best = gs.topk(keep, dim=-1).indices                                # [T, keep]
+        best = gs.sort(dim=-1, descending=True, stable=True).indices[:, :keep]     # ties: the lower index, as on the GPU
         ok = torch.zeros(T, groups, dtype=torch.bool, device=s.device).scatter_(1, best, True)
         sel = s.masked_fill(~ok.repeat_interleave(per, dim=1), -1.0)
     else:
         sel = s
-    ex = sel.topk(top, dim=-1).indices
+    ex = sel.sort(dim=-1, descending=True, stable=True).indices[:, :top]
     sc = s.gather(1, ex)
     return ex.to(torch.int32), (sc / (sc.sum(-1, keepdim=True) + WEIGHT_SUM_FLOOR) * scale).float()
 
