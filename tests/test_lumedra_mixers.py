@@ -221,6 +221,21 @@ def test_router_groups_shut_a_high_score_out(device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", ALL)
+def test_router_saturated_scores_are_told_apart(device, dtype):
+    """Logits of 12 and 12.001: their sigmoids differ by 6e-9, below what an f32 near 1 resolves, so a choice made on
+    f32 scores would tie them and take the lower index -- the better expert and the better group sit at the higher one."""
+    wr = torch.zeros(4, 8, dtype=torch.float64)
+    wr[:, 0] = torch.tensor([12.0, 12.0, 12.001, 12.0])
+    h = torch.zeros(2, 8, dtype=torch.float64)
+    h[:, 0] = 1.0
+    ex, _ = ops.router_topk(h.to(dtype).to(device), wr.float().to(device), 1, 1, 1, 1.0)
+    assert ex[:, 0].tolist() == [2, 2]
+    ex, wt = ops.router_topk(h.to(dtype).to(device), wr.float().to(device), 2, 2, 1, 1.0)      # groups (0, 1) and (2, 3)
+    assert sorted(ex[0].tolist()) == [2, 3] and abs(float(wt[0].sum()) - 1.0) < 1e-6
+    assert O.route(wr[:, 0], {"experts": 4, "top": 2, "groups": {"count": 2, "keep": 1}})[0] == [2, 3]
+
+
+@pytest.mark.parametrize("device,dtype", ALL)
 @pytest.mark.parametrize("W,top", [(36, 1), (256, 2), (1000, 3), (1024, 2), (2050, 2)])
 def test_stream_update_with_both_norms(W, top, device, dtype):
     g = torch.Generator().manual_seed(W)
