@@ -370,3 +370,54 @@ def test_served_through_the_model_manager(tmp_path):
     h = mgr.generator("lumedra-tiny")
     eng = h.engine
     assert isinstance(eng.model, LumedraModel) and eng.state_pool.num_slots == 4 and not eng.allocator.prefix_caching
+
+    async def both():
+        return await asyncio.gather(h.async_engine.generate([5, 6, 7, 8, 9, 10, 11], SamplingParams.greedy(5)),
+                                    h.async_engine.generate([3], SamplingParams.greedy(5)))
+
+    try:
+        seqs = asyncio.run(both())
+    finally:
+        h.async_engine.shutdown()
+    assert [len(s.output_ids) for s in seqs] == [5, 5]
+    assert eng.state_pool.num_free == 4
+    sd = {k: v.cpu() for k, v in eng.model.native_state_dict().items()}
+    for prompt, sq in zip(([5, 6, 7, 8, 9, 10, 11], [3]), seqs):
+        full = prompt + list(sq.output_ids)
+        lg = O.forward(eng.model.cfg.to_json(), sd, full[:-1])[len(prompt) - 1:]
+        assert [int(x) for x in lg.argmax(-1)] == list(sq.output_ids)
+
+
+@pytest.mark.gpu
+def test_pipelined_generation_on_captured_graphs():
+    """The server's step loop on the GPU in bf16: pipelined steps whose decode inputs are gathered on the device
+    from the previous step's ids, decode graphs replayed (router, experts, value blend and lightning state inside
+    them), three requests of different lengths that decode across a window's end; every token must be the oracle's
+    argmax for its prefix, or within a near tie."""
+    import asyncio
+
+    from llm_kubernetes_minikube_sharp4dev_amd.engine.llm_engine import AsyncLLMEngine
+
+    m, sd = model_and_weights("mid", "cuda", torch.bfloat16)
+    V = m.cfg.vocab_size
+    prompts = [toks(40, V, 70), toks(3, V, 71), toks(18, V, 72)]
+    eng = LLMEngine(m, None, block_size=16, max_model_len=256, max_num_seqs=4, num_blocks=24, eos_ids=set(),
+                    max_num_batched_tokens=32)
+    aeng = AsyncLLMEngine(eng)
+
+    async def run():
+        return await asyncio.gather(*[aeng.generate(p, SamplingParams.greedy(16)) for p in prompts])
+
+    try:
+        seqs = asyncio.run(run())
+    finally:
+        aeng.shutdown()
+    assert any(st.get("graph") is not None for st in eng.runner.graphs.values())
+    assert eng.state_pool.num_free == 4 and eng.allocator.num_free == 24
+    for p, sq in zip(prompts, seqs):
+        assert len(sq.output_ids) == 16
+        full = p + list(sq.output_ids)
+        lg = O.forward(CONFIGS["mid"], sd, full[:-1])[len(p) - 1:]
+        for i, tid in enumerate(sq.output_ids):
+            gap = float(lg[i].max() - lg[i, tid])
+            assert gap <= 0.25 * float(lg[i].max() - lg[i].min()), (i, gap)
